@@ -42,9 +42,66 @@ EXPORTS = [
 
 
 def build(jobs: int = 8) -> str:
-    """Compile the HIP sources for gfx950 (hipcc cross-compiles without a GPU)."""
+    """Compile the HIP sources for gfx950 (hipcc cross-compiles without a GPU): both libraries."""
     subprocess.check_call(["make", "-s", "-j%d" % jobs, "-C", CSRC])
     return LIB_PATH
+
+
+SEQ_LIB_PATH = os.environ.get("VLA_SEQ_LIB_PATH") or os.path.join(HERE, "libvla_seq_gfx950.so")
+SEQ_EXPORTS = [
+    "vla_seq_last_hip_error", "vla_seq_embed_positions", "vla_seq_scalar_rms_norm",
+    "vla_seq_residual_add", "vla_seq_poly_norm", "vla_seq_gated_head_rms_norm",
+    "vla_seq_key_cache_write", "vla_seq_window_attention", "vla_seq_gla_log_decay",
+    "vla_seq_gla_scan",
+]
+_seq_lib = None
+
+
+def build_seq(jobs: int = 8) -> str:
+    """Compile only csrc/seq_*.hip into libvla_seq_gfx950.so (include/vla_sequence_ops.h)."""
+    r = subprocess.run(["make", "-s", "-j%d" % jobs, "-C", CSRC, "seq"], stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building libvla_seq_gfx950.so failed:\n" + r.stdout[-4000:])
+    return SEQ_LIB_PATH
+
+
+def seq_lib():
+    """libvla_seq_gfx950.so, compiled first if it is not there (a fresh checkout serving a model
+    of the fp32-stream kind builds these few sources and nothing else)."""
+    global _seq_lib
+    if _seq_lib is None:
+        if not os.path.exists(SEQ_LIB_PATH):
+            build_seq()
+        import torch  # noqa: F401  (its HIP runtime first, as for lib())
+        L = C.CDLL(SEQ_LIB_PATH)
+        i, i64, f, p = C.c_int, C.c_int64, C.c_float, C.c_void_p
+        L.vla_seq_last_hip_error.argtypes = []
+        L.vla_seq_embed_positions.argtypes = [p, p, p, p, p, i, i, i, i, p]
+        L.vla_seq_scalar_rms_norm.argtypes = [p, p, p, p, p, f, i, i, i, p]
+        L.vla_seq_residual_add.argtypes = [p, p, i64, i, p]
+        L.vla_seq_poly_norm.argtypes = [p, i64, p, i64, p, f, i, i, i, p]
+        L.vla_seq_gated_head_rms_norm.argtypes = [p, i64, p, p, p, i64, f, f, i, i, i, i, p]
+        L.vla_seq_key_cache_write.argtypes = [p, p, i64, p, i, i, i, i, i, i, p]
+        L.vla_seq_window_attention.argtypes = [p, i64, p, i64, p, i64, p, p, i, p, p, p, i, i, i,
+                                               i, i, i, i, f, f, f, f, i, p]
+        L.vla_seq_gla_log_decay.argtypes = [p, p, i64, p, p, f, i, i, i, i, p]
+        L.vla_seq_gla_scan.argtypes = [p, p, i64, p, i64, p, i64, p, p, p, p, p, f, i, i, i, i, i,
+                                       i, p]
+        _seq_lib = L
+    return _seq_lib
+
+
+_SEQ_STATUS = {1: "Unsupported head size", 3: "Unsupported dtype", 5: "Invalid argument",
+               7: "HIP runtime error"}
+
+
+def seq_check(status: int, what: str) -> None:
+    if status != 0:
+        msg = _SEQ_STATUS.get(status, f"status {status}")
+        if status == 7:
+            msg += f" (hipError_t {seq_lib().vla_seq_last_hip_error()})"
+        raise RuntimeError(f"{what}: {msg}")
 
 
 TORCH_BINDING_NAME = "vla_torch_C"

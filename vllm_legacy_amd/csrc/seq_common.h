@@ -1,0 +1,45 @@
+// Shared by the sources of libvla_seq_gfx950.so: dtype dispatch, block reductions, error slot.
+#pragma once
+
+#include "../../include/vla_sequence_ops.h"
+#include "vla_common.h"
+
+namespace vla {
+namespace seq {
+
+void set_hip_error(int e);
+
+#define VLA_SEQ_HIP_CHECK(expr)          \
+  do {                                   \
+    hipError_t e_ = (expr);              \
+    if (e_ != hipSuccess) {              \
+      vla::seq::set_hip_error((int)e_);  \
+      return VLA_ERR_HIP;                \
+    }                                    \
+  } while (0)
+
+// calls f(S{}) with the scalar traits of a dtype code; VLA_ERR_DTYPE for an unknown code
+template <class F>
+inline int with_dtype(int dtype, F&& f) {
+  switch (dtype) {
+    case VLA_F16: return f(F16{});
+    case VLA_BF16: return f(BF16{});
+    case VLA_F32: return f(F32{});
+    default: return VLA_ERR_DTYPE;
+  }
+}
+
+// sum over a workgroup of up to 1024 threads; red holds 16 floats; every thread gets the sum
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  if (lane == 0) red[w] = v;
+  __syncthreads();
+  float r = 0.f;
+  for (int i = 0; i < nw; ++i) r += red[i];
+  __syncthreads();
+  return r;
+}
+
+}  // namespace seq
+}  // namespace vla

@@ -12,6 +12,7 @@ import torch
 import torch.nn as nn
 
 from vllm_legacy_amd import _custom_ops as ops
+from vllm_legacy_amd import _seq_ops as seq_ops
 from vllm_legacy_amd.distributed.communication_op import (
     PendingAllReduce, tensor_model_parallel_all_reduce_add_rms_norm)
 
@@ -78,4 +79,61 @@ class SiluAndMul(nn.Module):
         d = x.shape[-1] // 2
         out = torch.empty(x.shape[:-1] + (d, ), dtype=x.dtype, device=x.device)
         ops.silu_and_mul(out, x)
+        return out
+
+
+class ScalarRMSNorm(nn.Module):
+    """RMS norm of an fp32 residual stream with one gain for all coordinates:
+    out = x / sqrt(mean(x^2) + eps) * g, written in `out_dtype`.  add_rows ([T, W] fp32) and
+    add_row ([W] fp32) are added to the stream first, in place (the additions that open a pass
+    over looped layers ride in this launch)."""
+
+    def __init__(self, eps: float, device=None):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones((), dtype=torch.float32, device=device),
+                                   requires_grad=False)
+        self.variance_epsilon = float(eps)
+
+    def forward(self, x: torch.Tensor, out_dtype: torch.dtype, add_rows: Optional[torch.Tensor] = None,
+                add_row: Optional[torch.Tensor] = None) -> torch.Tensor:
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        seq_ops.scalar_rms_norm(out, x, self.weight.data.view(1), self.variance_epsilon, add_rows,
+                                add_row)
+        return out
+
+
+class PolyNorm(nn.Module):
+    """out = c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3, powers element by element, N(u) = u divided by
+    the root mean square of a token's vector u (eps inside the root)."""
+
+    def __init__(self, eps: float, device=None):
+        super().__init__()
+        self.weight = nn.Parameter(torch.tensor([1.0, 0.0, 0.0, 0.0], dtype=torch.float32,
+                                                device=device), requires_grad=False)
+        self.variance_epsilon = float(eps)
+
+    def forward(self, z: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if out is None:
+            out = torch.empty(z.shape, dtype=z.dtype, device=z.device)
+        seq_ops.poly_norm(out, z, self.weight.data, self.variance_epsilon)
+        return out
+
+
+class SinusoidalEmbedding(nn.Module):
+    """Token embedding plus the sinusoidal position vector (entry 2i sin, entry 2i + 1 cos of
+    p * base^(-2i / width)), written as the fp32 residual stream."""
+
+    def __init__(self, vocab_size: int, width: int, dtype=torch.bfloat16, device=None,
+                 base: float = 10000.0):
+        super().__init__()
+        self.weight = nn.Parameter(torch.zeros((vocab_size, width), dtype=dtype, device=device),
+                                   requires_grad=False)
+        i2 = torch.arange(0, width, 2, dtype=torch.float32)
+        inv_freq = torch.pow(torch.tensor(base, dtype=torch.float32), -i2 / width)
+        self.register_buffer("inv_freq", inv_freq.to(device), persistent=False)
+
+    def forward(self, input_ids: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        out = torch.empty((input_ids.numel(), self.weight.shape[1]), dtype=torch.float32,
+                          device=self.weight.device)
+        seq_ops.embed_positions(out, self.weight.data, input_ids, positions, self.inv_freq)
         return out
