@@ -102,6 +102,10 @@ class Scheduler:
             self.running.append(seq)
             step.append((seq, n))
             budget -= n
+        if not step and len(self.running) > 1:
+            # every running prompt is stuck behind the others' blocks: the newest starts over
+            self._preempt_last(self.running[0])
+            return self.schedule()
         return step
 
     def finish(self, seq: Sequence, reason: str) -> None:
