@@ -55,6 +55,14 @@ def parse():
     ap.add_argument("--rank-of", type=int, default=1,
                     help="kernel study: one process with the per-GPU shapes of an N-way tensor-"
                          "parallel rank (heads, FFN and vocabulary divided by N, no collectives)")
+    ap.add_argument("--arch", default=None, choices=["lusadra"],
+                    help="instead of the decode-step benchmark: prefill / decode throughput of this "
+                         "architecture beside the Llama stack at equal size, and its kernels beside "
+                         "the like kernels against their rooflines (tools/seq_arch_bench.py)")
+    ap.add_argument("--arch-size", default="2k", choices=["2k", "4k"])
+    ap.add_argument("--arch-prompt", type=int, default=4096)
+    ap.add_argument("--arch-batch", type=int, default=64)
+    ap.add_argument("--arch-context", type=int, default=4096)
     ap.add_argument("--attn-only", action="store_true",
                     help="time only the paged-attention launches (kernel study)")
     return ap.parse_args()
@@ -325,6 +333,11 @@ def launch_ranks(args) -> int:
 
 def main():
     args = parse()
+    if args.arch is not None:
+        assert args.gpus == 1, "--arch runs on one GPU"
+        from tools import seq_arch_bench
+        seq_arch_bench.run(args)
+        return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         sys.exit(launch_ranks(args))
     if os.environ.get("VLA_BENCH_WATCHDOG"):

@@ -120,17 +120,34 @@ class PagedKeys:
         # stale data everywhere: nothing may depend on a block being clean
         self.cache = (torch.randn(nb, block_size, G, D, generator=g) * 50).to(dtype).to(DEV)
 
-    def attend(self, q, k, gate, lo, hi, H, window, scale, slopes, coef=0.0, every=1.0, out_scale=1.0):
+    def attend(self, q, k, gate, lo, hi, H, window, scale, slopes, coef=0.0, every=1.0, out_scale=1.0,
+               kernel="auto"):
+        """kernel: "auto" (rows, picked per shape), "simple" (one wave per row and head), "tiles"
+        (matrix cores, 16-bit only)."""
         n = hi - lo
         pos = torch.arange(lo, hi)
         slots = (self.table[pos // self.bs].long() * self.bs + pos % self.bs).to(DEV)
         ops().key_cache_write(self.cache, k[lo:hi].to(DEV), slots)
         out = torch.empty(n, H * self.D, dtype=q.dtype, device=DEV)
+        sl = None if slopes is None else torch.tensor(slopes, dtype=torch.float32, device=DEV)
+        if kernel == "tiles":
+            i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)      # noqa: E731
+            ops().window_attention_tiles(out, q[lo:hi].to(DEV), None if gate is None else gate[lo:hi].to(DEV),
+                                         self.cache, self.table[None].contiguous().to(DEV), i32([0, n]), i32([lo]), n,
+                                         sl, H, window, scale, coef, every, out_scale)
+            return out.cpu()
+        ops().set_window_kernel(1 if kernel == "simple" else 0)
+        try:
+            self._rows(out, q, gate, lo, hi, pos, sl, H, window, scale, coef, every, out_scale)
+        finally:
+            ops().set_window_kernel(0)
+        return out.cpu()
+
+    def _rows(self, out, q, gate, lo, hi, pos, slopes_t, H, window, scale, coef, every, out_scale):
+        n = hi - lo
         ops().window_attention(out, q[lo:hi].to(DEV), None if gate is None else gate[lo:hi].to(DEV), self.cache,
                                self.table[None].contiguous().to(DEV), torch.zeros(n, dtype=torch.int32, device=DEV),
-                               pos.to(DEV), None if slopes is None else torch.tensor(slopes, dtype=torch.float32, device=DEV),
-                               H, window, scale, coef, every, out_scale)
-        return out.cpu()
+                               pos.to(DEV), slopes_t, H, window, scale, coef, every, out_scale)
 
 
 CASES = [  # H, G, D, window, block, n
@@ -144,8 +161,9 @@ CASES = [  # H, G, D, window, block, n
 ]
 
 
+@pytest.mark.parametrize("kernel", ["auto", "simple"])
 @pytest.mark.parametrize("H,G,D,window,bs,n", CASES)
-def test_window_attention_whole_portions_and_single_tokens(H, G, D, window, bs, n):
+def test_window_attention_whole_portions_and_single_tokens(H, G, D, window, bs, n, kernel):
     g = torch.Generator().manual_seed(n)
     q, k = torch.randn(n, H * D, generator=g), torch.randn(n, G * D, generator=g)
     gate = torch.randn(n, H * D, generator=g)
@@ -159,10 +177,78 @@ def test_window_attention_whole_portions_and_single_tokens(H, G, D, window, bs, 
         i = 0
         while lo < n:
             step = min(sizes[i % len(sizes)], n - lo)
-            got.append(pk.attend(q, k, gate, lo, lo + step, H, window, scale, slopes, coef, every, 0.6))
+            got.append(pk.attend(q, k, gate, lo, lo + step, H, window, scale, slopes, coef, every, 0.6, kernel))
             lo += step
             i += 1
         close(torch.cat(got), want, 3e-5)
+
+
+TILE_CASES = [  # H, G, D, window, block, n
+    (6, 2, 32, 7, 8, 70),
+    (3, 3, 96, 70, 16, 150),
+    (16, 2, 128, 33, 32, 100),    # eight query heads per KV head: two chunks of four
+    (4, 4, 64, 1, 4, 40),
+    (2, 1, 64, 0, 16, 90),
+    (5, 1, 128, 64, 16, 130),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("H,G,D,window,bs,n", TILE_CASES)
+def test_window_attention_tiles(H, G, D, window, bs, n, dtype):
+    """The matrix-core kernel on whole prompts and on portions that start anywhere (a tile's first
+    row in the middle of a page and of a window).  Inputs are 16-bit; the bar is the output's own
+    rounding (scores and weights are fp32 inside)."""
+    g = torch.Generator().manual_seed(n + H)
+    q, k = torch.randn(n, H * D, generator=g).to(dtype), torch.randn(n, G * D, generator=g).to(dtype)
+    gate = torch.randn(n, H * D, generator=g).to(dtype)
+    slopes, scale, coef, every = R.head_slopes(H), D**-0.5, 0.4, 3
+    want = R.windowed_key_attention(q.to(R.F), k.to(R.F), torch.arange(n), H, G, D, window, scale, coef, every, slopes)
+    want = want * torch.sigmoid(gate.to(R.F)) * 0.6
+    ulp = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
+    for sizes in ([n], [5, 33, 2, 40, 31, 32, 64]):
+        pk = PagedKeys(G, D, bs, n, dtype=dtype, seed=len(sizes))
+        got, lo, i = [], 0, 0
+        while lo < n:
+            step = min(sizes[i % len(sizes)], n - lo)
+            got.append(pk.attend(q, k, gate, lo, lo + step, H, window, scale, slopes, coef, every, 0.6, "tiles"))
+            lo += step
+            i += 1
+        close(torch.cat(got).float(), want, 1.5 * ulp)
+
+
+def test_window_attention_tiles_batch_matches_rows():
+    """Several sequences with contexts in one tiled launch against the row kernel on the same
+    cache: the two kernels differ by rounding only."""
+    H, G, D, bs, window = 8, 2, 64, 16, 37
+    lens, ctx = [70, 33, 5, 1], [10, 0, 64, 90]
+    g = torch.Generator().manual_seed(11)
+    total = [c + n for c, n in zip(ctx, lens)]
+    nb = sum((t + bs - 1) // bs for t in total)
+    perm = torch.randperm(nb, generator=g).tolist()
+    tables, at = [], 0
+    for t in total:
+        cnt = (t + bs - 1) // bs
+        tables.append(perm[at:at + cnt])
+        at += cnt
+    cache = torch.randn(nb, bs, G, D, generator=g).bfloat16().to(DEV)
+    T = sum(lens)
+    q = torch.randn(T, H * D, generator=g).bfloat16().to(DEV)
+    bt = torch.zeros(4, max(len(t) for t in tables), dtype=torch.int32)
+    for b, t in enumerate(tables):
+        bt[b, :len(t)] = torch.tensor(t, dtype=torch.int32)
+    starts = [0]
+    for n in lens:
+        starts.append(starts[-1] + n)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)      # noqa: E731
+    pos = torch.cat([torch.arange(c, c + n) for c, n in zip(ctx, lens)]).to(DEV)
+    tseq = torch.cat([torch.full((n, ), b, dtype=torch.int32) for b, n in enumerate(lens)]).to(DEV)
+    slopes = torch.tensor(R.head_slopes(H), dtype=torch.float32, device=DEV)
+    a, b_ = torch.empty_like(q), torch.empty_like(q)
+    ops().window_attention_tiles(a, q, None, cache, bt.to(DEV), i32(starts), i32(ctx), max(lens), slopes, H, window,
+                                 D**-0.5, 0.3, 16.0)
+    ops().window_attention(b_, q, None, cache, bt.to(DEV), tseq, pos, slopes, H, window, D**-0.5, 0.3, 16.0)
+    close(a.float(), b_.cpu().float(), 2.0**-7)
 
 
 def test_window_attention_without_bias_temperature_or_gate_in_bf16():
@@ -175,13 +261,14 @@ def test_window_attention_without_bias_temperature_or_gate_in_bf16():
     close(got.float(), want, 2.0**-8)
 
 
-@pytest.mark.parametrize("window,bs", [(5, 4), (16, 16), (17, 16), (64, 16), (65, 8), (100, 32)])
-@pytest.mark.parametrize("decode", [False, True])
+@pytest.mark.parametrize("window,bs", [(5, 4), (16, 16), (17, 16), (32, 16), (33, 8), (64, 16), (65, 8), (100, 32)])
+@pytest.mark.parametrize("decode", [False, True, "tiles"])
 def test_window_edge_decides_the_result(window, bs, decode):
     """Query i and key j share a long vector.  j = i - window + 1 is the last key inside: the
     result is that key.  j = i - window is the first outside: the result is far from it.  i is
     placed so that j falls on the first slot of a page, the last slot of a page, and position 0."""
-    H, G, D = 2, 1, 24
+    H, G, D = 2, 1, 32
+    dt = torch.bfloat16 if decode == "tiles" else torch.float32
     n = 3 * window + 2 * bs + 3
     scale = D**-0.5
     for inside in (True, False):
@@ -196,15 +283,21 @@ def test_window_edge_decides_the_result(window, bs, decode):
             big = math.sqrt((60.0 + window) / scale)        # score big^2 * scale outweighs any bias
             k[j] = u * big
             q[i] = (u * big).repeat(H)
-            pk = PagedKeys(G, D, bs, n, seed=j)
-            if decode:
+            q, k = q.to(dt), k.to(dt)
+            pk = PagedKeys(G, D, bs, n, dtype=dt, seed=j)
+            if decode == "tiles":
+                cut = max(1, i - 3)         # the portion's first tile starts three rows before i
+                pk.attend(q, k, None, 0, cut, H, window, scale, R.head_slopes(H), kernel="tiles")
+                out = pk.attend(q, k, None, cut, n, H, window, scale, R.head_slopes(H), kernel="tiles")[i - cut].float()
+                k = k.float()
+            elif decode:
                 pk.attend(q, k, None, 0, i, H, window, scale, R.head_slopes(H))
                 out = pk.attend(q, k, None, i, i + 1, H, window, scale, R.head_slopes(H))[0]
             else:
                 out = pk.attend(q, k, None, 0, n, H, window, scale, R.head_slopes(H))[i]
             for h in range(H):
                 d = float((out[h * D:(h + 1) * D] - k[j]).norm() / k[j].norm())
-                assert (d < 1e-3) if inside else (d > 0.5), (inside, i, j, h, d)
+                assert (d < (1e-2 if decode == "tiles" else 1e-3)) if inside else (d > 0.5), (inside, i, j, h, d)
 
 
 def test_query_temperature_steps_at_multiples_of_its_period():

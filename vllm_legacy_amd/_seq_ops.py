@@ -143,6 +143,43 @@ def window_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Te
             _dt(q.dtype), _stream(q.device)), "window_attention")
 
 
+def set_window_kernel(mode: int) -> None:
+    """0: window_attention picks its kernel per shape; 1: always one wave per (row, head)."""
+    seq_check(_lib.seq_lib().vla_seq_set_window_kernel(mode), "set_window_kernel")
+
+
+def window_attention_tiles_supported(q: torch.Tensor, head_dim: int) -> bool:
+    """Whether the matrix-core kernel for runs of query rows takes this query tensor."""
+    return bool(_lib.seq_lib().vla_seq_window_attention_tiles_supported(head_dim, _dt(q.dtype))) and \
+        q.data_ptr() % 8 == 0 and (q.stride(0) * q.element_size()) % 8 == 0
+
+
+def window_attention_tiles(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tensor],
+                           cache: torch.Tensor, block_tables: torch.Tensor, query_start_loc: torch.Tensor,
+                           context_lens: torch.Tensor, max_query_len: int, slopes: Optional[torch.Tensor],
+                           heads: int, window: int, scale: float, temp_coef: float = 0.0,
+                           temp_every: float = 1.0, out_scale: float = 1.0) -> None:
+    """The same attention as window_attention for 16-bit activations, tiled over runs of 32
+    query rows of a sequence (rows query_start_loc[b] .. of sequence b sit at positions
+    context_lens[b] ..)."""
+    _gpu(out, q, gate, cache, block_tables, query_start_loc, context_lens, slopes)
+    NB, BS, G, D = cache.shape
+    B = context_lens.numel()
+    assert cache.is_contiguous() and cache.dtype == q.dtype == out.dtype
+    for t in (block_tables, query_start_loc, context_lens):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    assert block_tables.dim() == 2 and block_tables.shape[0] == B and query_start_loc.numel() == B + 1
+    if slopes is not None:
+        assert slopes.dtype == torch.float32 and slopes.numel() == heads and slopes.is_contiguous()
+    with torch.cuda.device(q.device):
+        seq_check(_lib.seq_lib().vla_seq_window_attention_tiles(
+            out.data_ptr(), _rows(out, heads * D), q.data_ptr(), _rows(q, heads * D), _p(gate),
+            0 if gate is None else _rows(gate, heads * D), cache.data_ptr(), block_tables.data_ptr(),
+            block_tables.shape[1], query_start_loc.data_ptr(), context_lens.data_ptr(), _p(slopes), B,
+            int(max_query_len), heads, G, D, BS, NB, int(window), float(scale), float(temp_coef),
+            float(temp_every), float(out_scale), _dt(q.dtype), _stream(q.device)), "window_attention_tiles")
+
+
 def gla_log_decay(out: torch.Tensor, y: torch.Tensor, w2: torch.Tensor, bias: Optional[torch.Tensor],
                   inv_tau: float) -> None:
     """out fp32 [T, C] = ln(sigmoid(y @ w2^T + bias)) * inv_tau; y [T, R], w2 [C, R]."""

@@ -23,6 +23,8 @@ def geometric_slopes(num_heads: int, span: float = 8.0) -> List[float]:
 
 
 class WindowedKeyAttention(nn.Module):
+    # steps whose longest run of rows is at least this long take the tiled kernel (16-bit models)
+    TILE_MIN_QUERY = 4
 
     def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, scale: float,
                  window: Optional[int] = None, slopes: Optional[List[float]] = None,
@@ -46,7 +48,13 @@ class WindowedKeyAttention(nn.Module):
         """q, gate, out [T, H * D] and k [T, G * D]: views with free row strides.  Writes k into
         the cache, then attends; returns out (gated and scaled, in the activation dtype)."""
         ops.key_cache_write(cache, k, batch.slot_mapping)
-        ops.window_attention(out, q, gate, cache, batch.block_tables, batch.token_seq, batch.positions,
-                             self.slopes, self.num_heads, self.window, self.scale, self.temp_coef,
-                             self.temp_every, out_scale)
+        if batch.max_query_len >= self.TILE_MIN_QUERY and ops.window_attention_tiles_supported(q, self.head_dim):
+            # a step with runs of rows (prompts, portions): 32-row tiles on the matrix cores
+            ops.window_attention_tiles(out, q, gate, cache, batch.block_tables, batch.query_start_loc,
+                                       batch.context_lens, batch.max_query_len, self.slopes, self.num_heads,
+                                       self.window, self.scale, self.temp_coef, self.temp_every, out_scale)
+        else:
+            ops.window_attention(out, q, gate, cache, batch.block_tables, batch.token_seq, batch.positions,
+                                 self.slopes, self.num_heads, self.window, self.scale, self.temp_coef,
+                                 self.temp_every, out_scale)
         return out

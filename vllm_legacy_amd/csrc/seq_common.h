@@ -29,6 +29,15 @@ inline int with_dtype(int dtype, F&& f) {
   }
 }
 
+// Orders one wave's LDS traffic: what its lanes wrote before is visible to what they read after.
+// (The hardware keeps a wave's LDS instructions in order; the fences keep the compiler from
+// moving accesses of different types across the point.)
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // sum over a workgroup of up to 1024 threads; red holds 16 floats; every thread gets the sum
 __device__ __forceinline__ float block_sum(float v, float* red) {
   v = wave_sum(v);

@@ -14,11 +14,15 @@
 // max / sum (online softmax across tiles), then lane d accumulates sum_j p_j k_j[d] with
 // coalesced column reads.  The four waves of a workgroup take consecutive query heads of one
 // token, which share KV heads under grouped queries.
+#include <atomic>
+
 #include "seq_common.h"
 
 namespace vla {
 namespace seq {
 namespace {
+
+std::atomic<int> g_window_kernel{0};
 
 constexpr int kMaxDim = 256;
 constexpr int kAccum = kMaxDim / kWave;
@@ -57,7 +61,7 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void window_attention_kernel
   if (temp_coef != 0.f) qs *= 1.f + temp_coef * logf(floorf((float)(p + 1) / temp_every) + 1.f);
   for (int d = lane; d < dim; d += kWave)
     q_lds[w][d] = S::to_f32(q[(int64_t)t * q_stride + (int64_t)h * dim + d]) * qs;
-  __builtin_amdgcn_wave_barrier();
+  wave_sync();
   const float slope = slopes != nullptr ? slopes[h] : 0.f;
   const int64_t tok_stride = (int64_t)kv_heads * dim;
   // a block id outside the pool (a table the host filled wrongly) reads block 0 instead of faulting
@@ -85,9 +89,9 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void window_attention_kernel
     const float corr = expf(m - m_new);  // first tile: exp(-inf) = 0
     l = l * corr + wave_sum(pj);
     m = m_new;
-    __builtin_amdgcn_wave_barrier();
+    wave_sync();
     p_lds[w][lane] = pj;
-    __builtin_amdgcn_wave_barrier();
+    wave_sync();
 #pragma unroll
     for (int c = 0; c < kAccum; ++c) acc[c] *= corr;
     const int n = min(kWave, p - j0 + 1);
@@ -115,6 +119,376 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void window_attention_kernel
       out[(int64_t)t * out_stride + (int64_t)h * dim + d] = S::from_f32(v);
     }
   }
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// window_attention_group_kernel: one workgroup per (query row, KV head, chunk of up to kHeadChunk
+// query heads of that KV head).  For rows that come one per sequence (decode steps) the launch is
+// bound by reading each window once: the four waves split the window's 64-key tiles, each wave
+// copies its tile into LDS with coalesced 16-byte loads (once, for all heads of the chunk), lane j
+// scores key j against every head's query, the probabilities go through LDS, lane d accumulates
+// sum_j p_j k_j[d] from the same tile, and the waves' (max, sum, acc) are merged at the end.
+constexpr int kHeadChunk = 4;
+
+template <class S>
+__global__ __launch_bounds__(256) void window_attention_group_kernel(
+    typename S::T* __restrict__ out, int64_t out_stride, const typename S::T* __restrict__ q,
+    int64_t q_stride, const typename S::T* __restrict__ gate, int64_t gate_stride,
+    const typename S::T* __restrict__ cache, const int* __restrict__ block_tables, int max_blocks,
+    const int* __restrict__ token_seq, const int64_t* __restrict__ positions,
+    const float* __restrict__ slopes, int heads, int kv_heads, int dim, int block_size,
+    int num_blocks, int window, float scale, float temp_coef, float temp_every, float out_scale,
+    int row_pad) {
+  using T = typename S::T;
+  constexpr int VEC = 16 / sizeof(T);
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int row_len = dim + row_pad;                       // elements; rows stay 16-byte aligned
+  T* tiles = reinterpret_cast<T*>(smem);                   // [4][64][row_len]
+  float* q_lds = reinterpret_cast<float*>(smem + (size_t)4 * kWave * row_len * sizeof(T));  // [chunk][dim]
+  float* p_lds = q_lds + kHeadChunk * dim;                 // [4][64][chunk]
+  float* merge = p_lds + 4 * kWave * kHeadChunk;           // [4][chunk][2 + dim]
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int t = blockIdx.x;
+  const int group = heads / kv_heads;
+  const int chunks = (group + kHeadChunk - 1) / kHeadChunk;
+  const int g = blockIdx.y / chunks;
+  const int h0 = g * group + (blockIdx.y % chunks) * kHeadChunk;
+  const int nh = min(kHeadChunk, g * group + group - h0);
+  const int p = (int)positions[t];
+  const int* table = block_tables + (int64_t)token_seq[t] * max_blocks;
+  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  float qs = scale;
+  if (temp_coef != 0.f) qs *= 1.f + temp_coef * logf(floorf((float)(p + 1) / temp_every) + 1.f);
+  for (int i = threadIdx.x; i < nh * dim; i += 256)
+    q_lds[i] = S::to_f32(q[(int64_t)t * q_stride + (int64_t)h0 * dim + i]) * qs;
+  float slope[kHeadChunk];
+#pragma unroll
+  for (int hh = 0; hh < kHeadChunk; ++hh)
+    slope[hh] = (slopes != nullptr && hh < nh) ? slopes[h0 + hh] : 0.f;
+  __syncthreads();
+
+  T* tile = tiles + (size_t)w * kWave * row_len;
+  float* pw = p_lds + w * kWave * kHeadChunk;
+  const int64_t tok_stride = (int64_t)kv_heads * dim;
+  float m[kHeadChunk], l[kHeadChunk], acc[kHeadChunk][kAccum];
+#pragma unroll
+  for (int hh = 0; hh < kHeadChunk; ++hh) {
+    m[hh] = -INFINITY;
+    l[hh] = 0.f;
+#pragma unroll
+    for (int c = 0; c < kAccum; ++c) acc[hh][c] = 0.f;
+  }
+  const int vec_per_row = dim / VEC;   // dim % VEC == 0 is a launch condition
+  for (int j0 = lo + w * kWave; j0 <= p; j0 += 4 * kWave) {
+    const int n = min(kWave, p - j0 + 1);
+    // the tile: n rows of dim elements, 16 bytes per lane and load
+    for (int i = lane; i < n * vec_per_row; i += kWave) {
+      const int r = i / vec_per_row, v = i - r * vec_per_row;
+      const int j = j0 + r;
+      int b = table[j / block_size];
+      b = (unsigned)b < (unsigned)num_blocks ? b : 0;
+      const T* src = cache + ((int64_t)b * block_size + j % block_size) * tok_stride + (int64_t)g * dim + v * VEC;
+      *reinterpret_cast<u32x4*>(tile + (size_t)r * row_len + v * VEC) = *reinterpret_cast<const u32x4*>(src);
+    }
+    wave_sync();
+    // scores: lane = key
+    float s[kHeadChunk];
+#pragma unroll
+    for (int hh = 0; hh < kHeadChunk; ++hh) s[hh] = 0.f;
+    if (lane < n) {
+      const T* kr = tile + (size_t)lane * row_len;
+      for (int v = 0; v < vec_per_row; ++v) {
+        float kf[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) kf[e] = S::to_f32(kr[v * VEC + e]);
+#pragma unroll
+        for (int hh = 0; hh < kHeadChunk; ++hh) {
+          if (hh < nh) {
+            const float* qh = q_lds + hh * dim + v * VEC;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) s[hh] += qh[e] * kf[e];
+          }
+        }
+      }
+    }
+    const float dist = (float)(p - (j0 + lane));
+    float corr[kHeadChunk];
+#pragma unroll
+    for (int hh = 0; hh < kHeadChunk; ++hh) {
+      const float sv = lane < n ? s[hh] - slope[hh] * dist : -INFINITY;
+      const float m_new = fmaxf(m[hh], wave_max(sv));
+      const float pj = lane < n ? expf(sv - m_new) : 0.f;
+      corr[hh] = expf(m[hh] - m_new);
+      l[hh] = l[hh] * corr[hh] + wave_sum(pj);
+      m[hh] = m_new;
+      pw[lane * kHeadChunk + hh] = pj;
+    }
+    wave_sync();
+#pragma unroll
+    for (int hh = 0; hh < kHeadChunk; ++hh)
+#pragma unroll
+      for (int c = 0; c < kAccum; ++c) acc[hh][c] *= corr[hh];
+    for (int jj = 0; jj < n; ++jj) {
+      const f32x4 pv = *reinterpret_cast<const f32x4*>(pw + jj * kHeadChunk);
+#pragma unroll
+      for (int c = 0; c < kAccum; ++c) {
+        const int d = lane + c * kWave;
+        if (d < dim) {
+          const float kv = S::to_f32(tile[(size_t)jj * row_len + d]);
+#pragma unroll
+          for (int hh = 0; hh < kHeadChunk; ++hh) acc[hh][c] += pv[hh] * kv;
+        }
+      }
+    }
+    wave_sync();
+  }
+  // merge the four waves
+  float* mine = merge + (size_t)w * kHeadChunk * (2 + dim);
+#pragma unroll
+  for (int hh = 0; hh < kHeadChunk; ++hh) {
+    if (lane == 0) {
+      mine[hh * (2 + dim)] = m[hh];
+      mine[hh * (2 + dim) + 1] = l[hh];
+    }
+#pragma unroll
+    for (int c = 0; c < kAccum; ++c) {
+      const int d = lane + c * kWave;
+      if (d < dim) mine[hh * (2 + dim) + 2 + d] = acc[hh][c];
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < nh * dim; i += 256) {
+    const int hh = i / dim, d = i - hh * dim;
+    float mm = -INFINITY;
+    for (int ww = 0; ww < 4; ++ww) mm = fmaxf(mm, merge[((size_t)ww * kHeadChunk + hh) * (2 + dim)]);
+    float ll = 0.f, o = 0.f;
+    for (int ww = 0; ww < 4; ++ww) {
+      const float* src = merge + ((size_t)ww * kHeadChunk + hh) * (2 + dim);
+      const float f = src[0] == -INFINITY ? 0.f : expf(src[0] - mm);
+      ll += src[1] * f;
+      o += src[2 + d] * f;
+    }
+    float v = o * (out_scale / ll);
+    if (gate != nullptr) {
+      const float gv = S::to_f32(gate[(int64_t)t * gate_stride + (int64_t)(h0 + hh) * dim + d]);
+      v *= 1.f / (1.f + expf(-gv));
+    }
+    out[(int64_t)t * out_stride + (int64_t)(h0 + hh) * dim + d] = S::from_f32(v);
+  }
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// window_attention_tile_kernel<S, DB>: prompts and portions of prompts in 16-bit models, on the
+// matrix cores.  One workgroup per (sequence, tile of 32 consecutive query rows, KV head, chunk of
+// up to four of its query heads); wave w takes query head w of the chunk.  The keys from the
+// first row's window start to the last row walk through LDS in tiles of 32, staged once for all
+// waves, row-major for the first product and transposed for the second.  Both products run in
+// transposed form on 32x32x8 MFMAs, lane = (hf, c) = (lane >> 5, lane & 31):
+//   S^T = K q^T   A = K    lane: key c, dims 8 ks + 4 hf .. + 3
+//                 B = q^T  lane: query c, the same dims (registers, loaded once)
+//                 C        lane: query c, keys (i & 3) + 8 (i >> 2) + 4 hf, i = 0 .. 15
+//   O^T = K^T P^T A = K^T  lane: dim 32 n + c, keys 8 s + 4 hf .. + 3
+//                 B = P^T  lane: query c, the same keys = registers 4 s .. 4 s + 3 of C above
+//                 C        lane: query c, dims 32 n + (i & 3) + 8 (i >> 2) + 4 hf
+// so a lane owns one query's scores, running max / sum and output column; the softmax reduces
+// over registers and one exchange with the partner lane.  Scores leave the first product in fp32
+// and stay there; a weight enters the second product as the sum of two 16-bit numbers (its
+// rounding and the rounding of what the rounding lost), which keeps 16 bits of it and lets the
+// accumulation stay on the matrix cores.
+// Operands travel as two packed 32-bit words (four 16-bit values) and are cast to the builtin's
+// vector type at the call.
+template <class S>
+struct Mfma8;
+template <>
+struct Mfma8<BF16> {
+  typedef short V4 __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ f32x16 run(u32x2 a, u32x2 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(V4, a), __builtin_bit_cast(V4, b), c,
+                                                    0, 0, 0);
+  }
+};
+template <>
+struct Mfma8<F16> {
+  typedef _Float16 V4 __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ f32x16 run(u32x2 a, u32x2 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(V4, a), __builtin_bit_cast(V4, b), c, 0,
+                                                0, 0);
+  }
+};
+template <class S>
+__device__ __forceinline__ uint32_t bits16(float v) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, S::from_f32(v));
+}
+template <class S>
+__device__ __forceinline__ float from_bits16(uint32_t b) {
+  return S::to_f32(__builtin_bit_cast(typename S::T, (uint16_t)b));
+}
+
+constexpr int kTile = 32;
+
+template <class S, int DB>
+__global__ __launch_bounds__(256) void window_attention_tile_kernel(
+    typename S::T* __restrict__ out, int64_t out_stride, const typename S::T* __restrict__ q,
+    int64_t q_stride, const typename S::T* __restrict__ gate, int64_t gate_stride,
+    const typename S::T* __restrict__ cache, const int* __restrict__ block_tables, int max_blocks,
+    const int* __restrict__ query_start_loc, const int* __restrict__ context_lens,
+    const float* __restrict__ slopes, int heads, int kv_heads, int block_size, int num_blocks,
+    int window, float scale, float temp_coef, float temp_every, float out_scale) {
+  using T = typename S::T;
+  using M = Mfma8<S>;
+  constexpr int D = 32 * DB;
+  constexpr int KROW = D + 4, TROW = kTile + 4;      // elements; both keep 8-byte alignment
+  __shared__ __align__(16) T k_lds[kTile * KROW];    // [key][dim]
+  __shared__ __align__(16) T kt_lds[D * TROW];       // [dim][key]
+  const int b = blockIdx.z;
+  const int t0 = query_start_loc[b] + kTile * blockIdx.x;
+  const int nq = min(kTile, query_start_loc[b + 1] - t0);
+  if (nq <= 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int hf = lane >> 5, c = lane & 31;
+  const int group = heads / kv_heads;
+  const int chunks = (group + 3) / 4;
+  const int g = blockIdx.y / chunks;
+  const int h = g * group + (blockIdx.y % chunks) * 4 + w;
+  const bool active = h < g * group + group;
+  const int p0 = context_lens[b] + kTile * blockIdx.x, p_last = p0 + nq - 1;
+  const int j_lo = window > 0 ? max(0, p0 - window + 1) : 0;
+  const int* table = block_tables + (int64_t)b * max_blocks;
+  const int64_t tok_stride = (int64_t)kv_heads * D;
+  const int pq = p0 + c;
+  float qs = scale;
+  if (temp_coef != 0.f) qs *= 1.f + temp_coef * logf(floorf((float)(pq + 1) / temp_every) + 1.f);
+  const float slope = (slopes != nullptr && active) ? slopes[h] : 0.f;
+
+  u32x2 qf[D / 8];
+#pragma unroll
+  for (int ks = 0; ks < D / 8; ++ks) {
+    u32x2 v = {0u, 0u};
+    if (active && c < nq)
+      v = *reinterpret_cast<const u32x2*>(q + (int64_t)(t0 + c) * q_stride + (int64_t)h * D + 8 * ks + 4 * hf);
+    qf[ks] = v;
+  }
+  f32x16 o[DB];
+#pragma unroll
+  for (int n = 0; n < DB; ++n)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[n][i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  for (int j0 = j_lo; j0 <= p_last; j0 += kTile) {
+    __syncthreads();
+    for (int i = tid; i < kTile * (D / 4); i += 256) {
+      const int r = i / (D / 4), v = i - r * (D / 4);
+      const int j = j0 + r;
+      u32x2 x = {0u, 0u};
+      if (j <= p_last) {
+        int blk = table[j / block_size];
+        blk = (unsigned)blk < (unsigned)num_blocks ? blk : 0;
+        x = *reinterpret_cast<const u32x2*>(cache + ((int64_t)blk * block_size + j % block_size) * tok_stride +
+                                            (int64_t)g * D + 4 * v);
+      }
+      *reinterpret_cast<u32x2*>(k_lds + r * KROW + 4 * v) = x;
+      uint16_t* col = reinterpret_cast<uint16_t*>(kt_lds) + (4 * v) * TROW + r;
+      col[0] = (uint16_t)(x[0] & 0xffffu);
+      col[TROW] = (uint16_t)(x[0] >> 16);
+      col[2 * TROW] = (uint16_t)(x[1] & 0xffffu);
+      col[3 * TROW] = (uint16_t)(x[1] >> 16);
+    }
+    __syncthreads();
+    if (!active) continue;
+    f32x16 st;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) st[i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < D / 8; ++ks) {
+      const u32x2 a = *reinterpret_cast<const u32x2*>(k_lds + c * KROW + 8 * ks + 4 * hf);
+      st = M::run(a, qf[ks], st);
+    }
+    float mt = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int key = j0 + (i & 3) + 8 * (i >> 2) + 4 * hf;
+      const int dist = pq - key;
+      const bool ok = c < nq && dist >= 0 && (window <= 0 || dist < window);
+      st[i] = ok ? st[i] * qs - slope * (float)dist : -INFINITY;
+      mt = fmaxf(mt, st[i]);
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(m, mt);
+    const float corr = m_new == -INFINITY ? 1.f : expf(m - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      st[i] = m_new == -INFINITY ? 0.f : expf(st[i] - m_new);
+      psum += st[i];
+    }
+    l = l * corr + psum;          // this lane's keys; the partner's half is added at the end
+    m = m_new;
+#pragma unroll
+    for (int n = 0; n < DB; ++n)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[n][i] *= corr;
+#pragma unroll
+    for (int s8 = 0; s8 < 4; ++s8) {
+      uint32_t hb[4], lb[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float pv = st[4 * s8 + e];
+        hb[e] = bits16<S>(pv);
+        lb[e] = bits16<S>(pv - from_bits16<S>(hb[e]));
+      }
+      const u32x2 hi = {hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16)};
+      const u32x2 lo = {lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16)};
+#pragma unroll
+      for (int n = 0; n < DB; ++n) {
+        const u32x2 a = *reinterpret_cast<const u32x2*>(kt_lds + (32 * n + c) * TROW + 8 * s8 + 4 * hf);
+        o[n] = M::run(a, hi, o[n]);
+        o[n] = M::run(a, lo, o[n]);
+      }
+    }
+  }
+  if (!active) return;
+  l += __shfl_xor(l, 32, 64);
+  if (c >= nq) return;
+  const float inv = out_scale / l;
+#pragma unroll
+  for (int n = 0; n < DB; ++n)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int d = 32 * n + (i & 3) + 8 * (i >> 2) + 4 * hf;
+      float v = o[n][i] * inv;
+      if (gate != nullptr) {
+        const float gv = S::to_f32(gate[(int64_t)(t0 + c) * gate_stride + (int64_t)h * D + d]);
+        v *= 1.f / (1.f + expf(-gv));
+      }
+      out[(int64_t)(t0 + c) * out_stride + (int64_t)h * D + d] = S::from_f32(v);
+    }
+}
+
+template <class S>
+int launch_tiles(int db, dim3 grid, hipStream_t stream, typename S::T* out, int64_t out_stride,
+                 const typename S::T* q, int64_t q_stride, const typename S::T* gate,
+                 int64_t gate_stride, const typename S::T* cache, const int* block_tables,
+                 int max_blocks, const int* qsl, const int* ctx, const float* slopes, int heads,
+                 int kv_heads, int block_size, int num_blocks, int window, float scale,
+                 float temp_coef, float temp_every, float out_scale) {
+#define VLA_TILE(DB)                                                                             \
+  window_attention_tile_kernel<S, DB><<<grid, 256, 0, stream>>>(                                 \
+      out, out_stride, q, q_stride, gate, gate_stride, cache, block_tables, max_blocks, qsl, ctx, \
+      slopes, heads, kv_heads, block_size, num_blocks, window, scale, temp_coef, temp_every,     \
+      out_scale)
+  switch (db) {
+    case 1: VLA_TILE(1); break;
+    case 2: VLA_TILE(2); break;
+    case 3: VLA_TILE(3); break;
+    case 4: VLA_TILE(4); break;
+    default: return VLA_ERR_HEAD_SIZE;
+  }
+#undef VLA_TILE
+  VLA_SEQ_HIP_CHECK(hipGetLastError());
+  return VLA_OK;
 }
 
 }  // namespace
@@ -160,13 +534,77 @@ extern "C" int vla_seq_window_attention(void* out, int64_t out_stride, const voi
   if (dim <= 0 || dim > kMaxDim) return VLA_ERR_HEAD_SIZE;
   return with_dtype(dtype, [&](auto s) {
     using S = decltype(s);
+    using T = typename S::T;
+    constexpr int VEC = 16 / sizeof(T);
+    // the grouped kernel wants 16-byte rows everywhere it loads vectors and its tiles in LDS
+    const int row_pad = VEC;
+    const size_t lds = (size_t)4 * kWave * (dim + row_pad) * sizeof(T) +
+                       sizeof(float) * ((size_t)kHeadChunk * dim + 4 * kWave * kHeadChunk +
+                                        (size_t)4 * kHeadChunk * (2 + dim));
+    const bool grouped = g_window_kernel.load(std::memory_order_relaxed) != 1 && dim % VEC == 0 &&
+                         ((uintptr_t)cache % 16) == 0 && lds <= 150 * 1024;
+    if (grouped) {
+      const int group = heads / kv_heads;
+      const dim3 grid(num_tokens, kv_heads * ((group + kHeadChunk - 1) / kHeadChunk));
+      if (lds > 64 * 1024)
+        VLA_SEQ_HIP_CHECK(hipFuncSetAttribute(
+            reinterpret_cast<const void*>(&window_attention_group_kernel<S>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      window_attention_group_kernel<S><<<grid, 256, lds, (hipStream_t)stream>>>(
+          (T*)out, out_stride, (const T*)q, q_stride, (const T*)gate, gate_stride, (const T*)cache,
+          block_tables, max_blocks, token_seq, positions, slopes, heads, kv_heads, dim, block_size,
+          num_blocks, window, scale, temp_coef, temp_every, out_scale, row_pad);
+      VLA_SEQ_HIP_CHECK(hipGetLastError());
+      return VLA_OK;
+    }
     const dim3 grid((heads + kHeadsPerGroup - 1) / kHeadsPerGroup, num_tokens);
     window_attention_kernel<S><<<grid, kWave * kHeadsPerGroup, 0, (hipStream_t)stream>>>(
-        (typename S::T*)out, out_stride, (const typename S::T*)q, q_stride,
-        (const typename S::T*)gate, gate_stride, (const typename S::T*)cache, block_tables,
-        max_blocks, token_seq, positions, slopes, heads, kv_heads, dim, block_size, num_blocks, window,
-        scale, temp_coef, temp_every, out_scale);
+        (T*)out, out_stride, (const T*)q, q_stride, (const T*)gate, gate_stride, (const T*)cache,
+        block_tables, max_blocks, token_seq, positions, slopes, heads, kv_heads, dim, block_size,
+        num_blocks, window, scale, temp_coef, temp_every, out_scale);
     VLA_SEQ_HIP_CHECK(hipGetLastError());
     return VLA_OK;
   });
+}
+
+// 0: pick per shape; 1: the one-wave-per-(row, head) kernel; (tests run both)
+extern "C" int vla_seq_set_window_kernel(int mode) {
+  if (mode < 0 || mode > 2) return VLA_ERR_ARG;
+  g_window_kernel.store(mode, std::memory_order_relaxed);
+  return VLA_OK;
+}
+
+extern "C" int vla_seq_window_attention_tiles_supported(int dim, int dtype) {
+  return (dtype == VLA_F16 || dtype == VLA_BF16) && dim % 32 == 0 && dim >= 32 && dim <= 128;
+}
+
+extern "C" int vla_seq_window_attention_tiles(
+    void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* gate,
+    int64_t gate_stride, const void* cache, const int* block_tables, int max_blocks,
+    const int* query_start_loc, const int* context_lens, const float* slopes, int num_seqs,
+    int max_query_len, int heads, int kv_heads, int dim, int block_size, int num_blocks, int window,
+    float scale, float temp_coef, float temp_every, float out_scale, int dtype, void* stream) {
+  if (num_seqs == 0 || max_query_len == 0) return VLA_OK;
+  if (!out || !q || !cache || !block_tables || !query_start_loc || !context_lens || num_seqs < 0 ||
+      max_query_len < 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || block_size <= 0 ||
+      num_blocks <= 0 || max_blocks <= 0 || out_stride < (int64_t)heads * dim ||
+      q_stride < (int64_t)heads * dim || (gate && gate_stride < (int64_t)heads * dim) ||
+      (temp_coef != 0.f && !(temp_every > 0.f)))
+    return VLA_ERR_ARG;
+  if (!vla_seq_window_attention_tiles_supported(dim, dtype)) return VLA_ERR_HEAD_SIZE;
+  // 8-byte fragment loads: query rows and cache rows must allow them
+  if (((uintptr_t)q % 8) || ((q_stride * 2) % 8) || ((uintptr_t)cache % 8)) return VLA_ERR_ARG;
+  const int group = heads / kv_heads;
+  const dim3 grid((max_query_len + kTile - 1) / kTile, kv_heads * ((group + 3) / 4), num_seqs);
+  if (dtype == VLA_BF16)
+    return launch_tiles<BF16>(dim / 32, grid, (hipStream_t)stream, (__bf16*)out, out_stride,
+                              (const __bf16*)q, q_stride, (const __bf16*)gate, gate_stride,
+                              (const __bf16*)cache, block_tables, max_blocks, query_start_loc,
+                              context_lens, slopes, heads, kv_heads, block_size, num_blocks, window,
+                              scale, temp_coef, temp_every, out_scale);
+  return launch_tiles<F16>(dim / 32, grid, (hipStream_t)stream, (_Float16*)out, out_stride,
+                           (const _Float16*)q, q_stride, (const _Float16*)gate, gate_stride,
+                           (const _Float16*)cache, block_tables, max_blocks, query_start_loc,
+                           context_lens, slopes, heads, kv_heads, block_size, num_blocks, window, scale,
+                           temp_coef, temp_every, out_scale);
 }
