@@ -89,12 +89,32 @@ int vla_seq_gla_log_decay(float* out, const void* y, int64_t y_stride, const voi
  * per head, S [dim, vdim].  Sequence b starts from zero when context_lens[b] == 0 and from
  * state[state_slots[b]] otherwise, and leaves its state there.  q, k [T, heads * dim] and
  * v [T, heads * vdim] `dtype` with strides, log_decay fp32 [T, heads * dim], o fp32
- * [T, heads, vdim], state fp32 [num_slots, heads, dim, vdim]. */
+ * [T, heads, vdim], state fp32 [num_slots, heads, dim, vdim].  max_query_len: the longest run of
+ * rows of one sequence in the step, or 0 if unknown (a hint that sizes the staging buffers). */
 int vla_seq_gla_scan(float* o, const void* q, int64_t q_stride, const void* k, int64_t k_stride,
                      const void* v, int64_t v_stride, const float* log_decay, float* state,
                      const int* query_start_loc, const int* context_lens, const int* state_slots,
-                     float q_scale, int num_seqs, int num_slots, int heads, int dim, int vdim,
-                     int dtype, void* stream);
+                     float q_scale, int num_seqs, int num_slots, int max_query_len, int heads,
+                     int dim, int vdim, int dtype, void* stream);
+
+/* The same attention for 16-bit activations, tiled over runs of 32 query rows of a sequence on
+ * the matrix cores: rows query_start_loc[b] .. query_start_loc[b + 1] - 1 of sequence b sit at
+ * positions context_lens[b] ...  dim must be a multiple of 32, at most 128
+ * (vla_seq_window_attention_tiles_supported); query rows and cache rows must be 8-byte aligned. */
+int vla_seq_window_attention_tiles_supported(int dim, int dtype);
+int vla_seq_window_attention_tiles(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                   const void* gate, int64_t gate_stride, const void* cache,
+                                   const int* block_tables, int max_blocks,
+                                   const int* query_start_loc, const int* context_lens,
+                                   const float* slopes, int num_seqs, int max_query_len, int heads,
+                                   int kv_heads, int dim, int block_size, int num_blocks,
+                                   int window, float scale, float temp_coef, float temp_every,
+                                   float out_scale, int dtype, void* stream);
+
+/* Kernel choice for tests: window attention 0 = per shape, 1 = one wave per (row, head);
+ * scan 0 = per shape, 1 = token by token. */
+int vla_seq_set_window_kernel(int mode);
+int vla_seq_set_scan_kernel(int mode);
 
 #ifdef __cplusplus
 }

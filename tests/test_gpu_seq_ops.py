@@ -375,11 +375,26 @@ def test_gla_log_decay(C, rank, dtype):
     assert bool((out <= 0).all())
 
 
+SCAN_KERNEL = {"mode": 0}      # 0: picked per shape (the blocked walk where it fits); 1: token by token
+
+
+@pytest.fixture(params=[0, 1], ids=["blocked", "token-by-token"])
+def scan_kernel(request):
+    SCAN_KERNEL["mode"] = request.param
+    yield request.param
+    SCAN_KERNEL["mode"] = 0
+
+
 def run_scan(q, k, v, ln_a, state, starts, ctx, slots, H, D, V, q_scale):
     T = q.shape[0]
     o = torch.empty(T, H, V, dtype=torch.float32, device=DEV)
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)      # noqa: E731
-    ops().gla_scan(o, q.to(DEV), k.to(DEV), v.to(DEV), ln_a.to(DEV), state, i32(starts), i32(ctx), i32(slots), q_scale)
+    ops().set_scan_kernel(SCAN_KERNEL["mode"])
+    try:
+        ops().gla_scan(o, q.to(DEV), k.to(DEV), v.to(DEV), ln_a.to(DEV), state, i32(starts), i32(ctx), i32(slots),
+                       q_scale)
+    finally:
+        ops().set_scan_kernel(0)
     return o.cpu()
 
 
@@ -387,13 +402,13 @@ SCAN = [(2, 8, 16), (3, 32, 64), (1, 5, 7), (2, 64, 128), (2, 100, 40), (1, 16, 
 
 
 @pytest.mark.parametrize("H,D,V", SCAN)
-def test_gla_scan_whole_portions_and_single_tokens(H, D, V):
-    n = 37
+def test_gla_scan_whole_portions_and_single_tokens(H, D, V, scan_kernel):
+    n = 57
     g = torch.Generator().manual_seed(H * D + V)
     q, k, v = torch.randn(n, H * D, generator=g), torch.randn(n, H * D, generator=g), torch.randn(n, H * V, generator=g)
     ln_a = -torch.rand(n, H * D, generator=g) * 0.3
     want, want_state = R.gated_linear_attention(q.to(R.F) * 0.37, k.to(R.F), v.to(R.F), ln_a.to(R.F), H, D, V)
-    for sizes in ([n], [2, 5, 1, 1, 9, 3], [1] * n):
+    for sizes in ([n], [2, 5, 1, 1, 19, 3, 16, 17], [1] * n):
         state = torch.full((3, H, D, V), 7.0, device=DEV)     # stale: the sequence starts at context 0
         got, lo, i = [], 0, 0
         while lo < n:
@@ -407,12 +422,12 @@ def test_gla_scan_whole_portions_and_single_tokens(H, D, V):
         assert float((state[0] - 7).abs().max()) == 0 and float((state[2] - 7).abs().max()) == 0
 
 
-def test_gla_scan_batch_with_slots_used_again():
+def test_gla_scan_batch_with_slots_used_again(scan_kernel):
     """Four sequences of unequal length in one launch, two of them continuing; then the slot of a
     finished one goes to a new sequence, which must not see what the slot held."""
     H, D, V = 2, 12, 20
     g = torch.Generator().manual_seed(9)
-    lens = [9, 1, 14, 5]
+    lens = [9, 1, 34, 5]
 
     def mk(n):
         return (torch.randn(n, H * D, generator=g), torch.randn(n, H * D, generator=g),
@@ -440,7 +455,7 @@ def test_gla_scan_batch_with_slots_used_again():
 
 
 @pytest.mark.parametrize("decode", [False, True])
-def test_gla_carries_a_far_token(decode):
+def test_gla_carries_a_far_token(decode, scan_kernel):
     """One channel never decays and holds a key at token 3 only; 600 tokens later a query on
     that channel returns token 3's value, through one launch or through 600."""
     H, D, V, n = 1, 8, 16, 604

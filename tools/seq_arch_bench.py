@@ -115,9 +115,15 @@ def run(args):
             k = torch.randn(T, G * D, device=dev, dtype=dt)
             gate = torch.randn(T, H * D, device=dev, dtype=dt)
             out = torch.empty_like(q)
-            sec = timed(lambda: sops.window_attention(out, q, gate, keys, batch.block_tables, batch.token_seq,
-                                                      batch.positions, lay.attn.slopes, H, W, D**-0.5, 0.3, 512.0, 0.5),
-                        5 if tag == "prefill" else 20)
+            if tag == "prefill":     # runs of rows: the tiled kernel, as the layer picks it
+                sec = timed(lambda: sops.window_attention_tiles(out, q, gate, keys, batch.block_tables,
+                                                                batch.query_start_loc, batch.context_lens,
+                                                                batch.max_query_len, lay.attn.slopes, H, W, D**-0.5,
+                                                                0.3, 512.0, 0.5), 5)
+            else:
+                sec = timed(lambda: sops.window_attention(out, q, gate, keys, batch.block_tables, batch.token_seq,
+                                                          batch.positions, lay.attn.slopes, H, W, D**-0.5, 0.3, 512.0,
+                                                          0.5), 20)
             if tag == "prefill":
                 pairs = sum(min(W, p + 1) for p in range(T))
                 record(kern, "lusadra.window_attention.prefill", sec, flops=4.0 * pairs * H * D,
@@ -132,7 +138,8 @@ def run(args):
             ld = -torch.rand(T, Hr * Dr, device=dev) * 0.1
             o = torch.empty(T, Hr, Vr, device=dev)
             sec = timed(lambda: sops.gla_scan(o, qr, kr, vr, ld, state, batch.query_start_loc, batch.context_lens,
-                                              batch.state_slots, Dr**-0.5), 5 if tag == "prefill" else 20)
+                                              batch.state_slots, Dr**-0.5, batch.max_query_len),
+                        5 if tag == "prefill" else 20)
             nseq = batch.num_seqs
             record(kern, f"lusadra.gla_scan.{tag}", sec, peak=FMA_F32, flops=4.0 * T * Hr * Dr * Vr,
                    nbytes=T * (2.0 * (2 * Hr * Dr + Hr * Vr) + 4.0 * Hr * Dr + 4.0 * Hr * Vr) + 8.0 * nseq * Hr * Dr * Vr,

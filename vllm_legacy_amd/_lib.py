@@ -53,7 +53,7 @@ SEQ_EXPORTS = [
     "vla_seq_residual_add", "vla_seq_poly_norm", "vla_seq_gated_head_rms_norm",
     "vla_seq_key_cache_write", "vla_seq_window_attention", "vla_seq_gla_log_decay",
     "vla_seq_gla_scan", "vla_seq_set_window_kernel", "vla_seq_window_attention_tiles",
-    "vla_seq_window_attention_tiles_supported",
+    "vla_seq_window_attention_tiles_supported", "vla_seq_set_scan_kernel",
 ]
 _seq_lib = None
 
@@ -87,12 +87,13 @@ def seq_lib():
         L.vla_seq_window_attention.argtypes = [p, i64, p, i64, p, i64, p, p, i, p, p, p, i, i, i,
                                                i, i, i, i, f, f, f, f, i, p]
         L.vla_seq_set_window_kernel.argtypes = [i]
+        L.vla_seq_set_scan_kernel.argtypes = [i]
         L.vla_seq_window_attention_tiles_supported.argtypes = [i, i]
         L.vla_seq_window_attention_tiles.argtypes = [p, i64, p, i64, p, i64, p, p, i, p, p, p, i, i, i,
                                                      i, i, i, i, i, f, f, f, f, i, p]
         L.vla_seq_gla_log_decay.argtypes = [p, p, i64, p, p, f, i, i, i, i, p]
         L.vla_seq_gla_scan.argtypes = [p, p, i64, p, i64, p, i64, p, p, p, p, p, f, i, i, i, i, i,
-                                       i, p]
+                                       i, i, p]
         _seq_lib = L
     return _seq_lib
 

@@ -148,6 +148,11 @@ def set_window_kernel(mode: int) -> None:
     seq_check(_lib.seq_lib().vla_seq_set_window_kernel(mode), "set_window_kernel")
 
 
+def set_scan_kernel(mode: int) -> None:
+    """0: gla_scan picks its kernel per shape; 1: always the token-by-token kernel."""
+    seq_check(_lib.seq_lib().vla_seq_set_scan_kernel(mode), "set_scan_kernel")
+
+
 def window_attention_tiles_supported(q: torch.Tensor, head_dim: int) -> bool:
     """Whether the matrix-core kernel for runs of query rows takes this query tensor."""
     return bool(_lib.seq_lib().vla_seq_window_attention_tiles_supported(head_dim, _dt(q.dtype))) and \
@@ -198,7 +203,7 @@ def gla_log_decay(out: torch.Tensor, y: torch.Tensor, w2: torch.Tensor, bias: Op
 
 def gla_scan(o: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, log_decay: torch.Tensor,
              state: torch.Tensor, query_start_loc: torch.Tensor, context_lens: torch.Tensor,
-             state_slots: torch.Tensor, q_scale: float) -> None:
+             state_slots: torch.Tensor, q_scale: float, max_query_len: int = 0) -> None:
     """o fp32 [T, H, V]; q, k [T, H*D]; v [T, H*V]; log_decay fp32 [T, H*D]; state fp32
     [slots, H, D, V]; query_start_loc int32 [B+1], context_lens / state_slots int32 [B]."""
     _gpu(o, q, k, v, log_decay, state, query_start_loc, context_lens, state_slots)
@@ -216,5 +221,5 @@ def gla_scan(o: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
         seq_check(_lib.seq_lib().vla_seq_gla_scan(
             o.data_ptr(), q.data_ptr(), _rows(q, H * D), k.data_ptr(), _rows(k, H * D), v.data_ptr(),
             _rows(v, H * V), log_decay.data_ptr(), state.data_ptr(), query_start_loc.data_ptr(),
-            context_lens.data_ptr(), state_slots.data_ptr(), float(q_scale), B, slots, H, D, V,
+            context_lens.data_ptr(), state_slots.data_ptr(), float(q_scale), B, slots, int(max_query_len), H, D, V,
             _dt(q.dtype), _stream(q.device)), "gla_scan")

@@ -41,6 +41,6 @@ class GatedLinearRecurrence(nn.Module):
         ops.gla_log_decay(log_decay, y, w2, bias, self.inv_tau)
         o = torch.empty((T, H, V), dtype=torch.float32, device=q.device)
         ops.gla_scan(o, q, k, v, log_decay, state, batch.query_start_loc, batch.context_lens,
-                     batch.state_slots, self.q_scale)
+                     batch.state_slots, self.q_scale, batch.max_query_len)
         ops.gated_head_rms_norm(out, o, norm_weight, gate, self.eps, out_scale)
         return out

@@ -127,9 +127,21 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void window_attention_kernel
 // query heads of that KV head).  For rows that come one per sequence (decode steps) the launch is
 // bound by reading each window once: the four waves split the window's 64-key tiles, each wave
 // copies its tile into LDS with coalesced 16-byte loads (once, for all heads of the chunk), lane j
-// scores key j against every head's query, the probabilities go through LDS, lane d accumulates
-// sum_j p_j k_j[d] from the same tile, and the waves' (max, sum, acc) are merged at the end.
+// scores key j against every head's query, the probabilities go through LDS, every lane
+// accumulates two neighbouring dims of sum_j p_j k_j from the same tile, and the waves' (max, sum,
+// acc) are merged at the end.  The queries are read through wave-uniform addresses, so they sit
+// in scalar registers and the score loop's only LDS traffic is the key row.
 constexpr int kHeadChunk = 4;
+constexpr int kPairs = kMaxDim / (2 * kWave);   // passes of 128 dims in the weighted sum
+
+template <class S>
+__device__ __forceinline__ float lo16(uint32_t w) {
+  return S::to_f32(__builtin_bit_cast(typename S::T, (uint16_t)(w & 0xffffu)));
+}
+template <class S>
+__device__ __forceinline__ float hi16(uint32_t w) {
+  return S::to_f32(__builtin_bit_cast(typename S::T, (uint16_t)(w >> 16)));
+}
 
 template <class S>
 __global__ __launch_bounds__(256) void window_attention_group_kernel(
@@ -145,8 +157,7 @@ __global__ __launch_bounds__(256) void window_attention_group_kernel(
   extern __shared__ __align__(16) unsigned char smem[];
   const int row_len = dim + row_pad;                       // elements; rows stay 16-byte aligned
   T* tiles = reinterpret_cast<T*>(smem);                   // [4][64][row_len]
-  float* q_lds = reinterpret_cast<float*>(smem + (size_t)4 * kWave * row_len * sizeof(T));  // [chunk][dim]
-  float* p_lds = q_lds + kHeadChunk * dim;                 // [4][64][chunk]
+  float* p_lds = reinterpret_cast<float*>(smem + (size_t)4 * kWave * row_len * sizeof(T));  // [4][64][chunk]
   float* merge = p_lds + 4 * kWave * kHeadChunk;           // [4][chunk][2 + dim]
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int t = blockIdx.x;
@@ -160,24 +171,26 @@ __global__ __launch_bounds__(256) void window_attention_group_kernel(
   const int lo = window > 0 ? max(0, p - window + 1) : 0;
   float qs = scale;
   if (temp_coef != 0.f) qs *= 1.f + temp_coef * logf(floorf((float)(p + 1) / temp_every) + 1.f);
-  for (int i = threadIdx.x; i < nh * dim; i += 256)
-    q_lds[i] = S::to_f32(q[(int64_t)t * q_stride + (int64_t)h0 * dim + i]) * qs;
+  // heads past the chunk's last read the last one's query again (their results are dropped)
+  const T* qrow[kHeadChunk];
   float slope[kHeadChunk];
 #pragma unroll
-  for (int hh = 0; hh < kHeadChunk; ++hh)
-    slope[hh] = (slopes != nullptr && hh < nh) ? slopes[h0 + hh] : 0.f;
-  __syncthreads();
+  for (int hh = 0; hh < kHeadChunk; ++hh) {
+    const int h = h0 + min(hh, nh - 1);
+    qrow[hh] = q + (int64_t)t * q_stride + (int64_t)h * dim;
+    slope[hh] = slopes != nullptr ? slopes[h] : 0.f;
+  }
 
   T* tile = tiles + (size_t)w * kWave * row_len;
   float* pw = p_lds + w * kWave * kHeadChunk;
   const int64_t tok_stride = (int64_t)kv_heads * dim;
-  float m[kHeadChunk], l[kHeadChunk], acc[kHeadChunk][kAccum];
+  float m[kHeadChunk], l[kHeadChunk], acc[kHeadChunk][kPairs][2];
 #pragma unroll
   for (int hh = 0; hh < kHeadChunk; ++hh) {
     m[hh] = -INFINITY;
     l[hh] = 0.f;
 #pragma unroll
-    for (int c = 0; c < kAccum; ++c) acc[hh][c] = 0.f;
+    for (int c = 0; c < kPairs; ++c) acc[hh][c][0] = acc[hh][c][1] = 0.f;
   }
   const int vec_per_row = dim / VEC;   // dim % VEC == 0 is a launch condition
   for (int j0 = lo + w * kWave; j0 <= p; j0 += 4 * kWave) {
@@ -192,31 +205,32 @@ __global__ __launch_bounds__(256) void window_attention_group_kernel(
       *reinterpret_cast<u32x4*>(tile + (size_t)r * row_len + v * VEC) = *reinterpret_cast<const u32x4*>(src);
     }
     wave_sync();
-    // scores: lane = key
+    // scores: lane = key; its row comes from LDS 16 bytes at a time, the queries from scalar loads
     float s[kHeadChunk];
 #pragma unroll
     for (int hh = 0; hh < kHeadChunk; ++hh) s[hh] = 0.f;
-    if (lane < n) {
-      const T* kr = tile + (size_t)lane * row_len;
-      for (int v = 0; v < vec_per_row; ++v) {
-        float kf[VEC];
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) kf[e] = S::to_f32(kr[v * VEC + e]);
-#pragma unroll
-        for (int hh = 0; hh < kHeadChunk; ++hh) {
-          if (hh < nh) {
-            const float* qh = q_lds + hh * dim + v * VEC;
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) s[hh] += qh[e] * kf[e];
-          }
-        }
+    const T* kr = tile + (size_t)min(lane, n - 1) * row_len;
+    // (rows are read 4 bytes at a time: wider reads of lane-strided rows came back wrong on the
+    // part, so the row costs dim / 2 reads in 16-bit models; the arithmetic still dominates)
+    for (int d = 0; d < dim; d += 2) {
+      float k0, k1;
+      if constexpr (sizeof(T) == 4) {
+        k0 = kr[d];
+        k1 = kr[d + 1];
+      } else {
+        const uint32_t kk = *reinterpret_cast<const uint32_t*>(kr + d);
+        k0 = lo16<S>(kk);
+        k1 = hi16<S>(kk);
       }
+#pragma unroll
+      for (int hh = 0; hh < kHeadChunk; ++hh)      // the same address in every lane: scalar loads
+        s[hh] += S::to_f32(qrow[hh][d]) * k0 + S::to_f32(qrow[hh][d + 1]) * k1;
     }
     const float dist = (float)(p - (j0 + lane));
     float corr[kHeadChunk];
 #pragma unroll
     for (int hh = 0; hh < kHeadChunk; ++hh) {
-      const float sv = lane < n ? s[hh] - slope[hh] * dist : -INFINITY;
+      const float sv = lane < n ? s[hh] * qs - slope[hh] * dist : -INFINITY;
       const float m_new = fmaxf(m[hh], wave_max(sv));
       const float pj = lane < n ? expf(sv - m_new) : 0.f;
       corr[hh] = expf(m[hh] - m_new);
@@ -228,16 +242,33 @@ __global__ __launch_bounds__(256) void window_attention_group_kernel(
 #pragma unroll
     for (int hh = 0; hh < kHeadChunk; ++hh)
 #pragma unroll
-      for (int c = 0; c < kAccum; ++c) acc[hh][c] *= corr[hh];
+      for (int c = 0; c < kPairs; ++c) {
+        acc[hh][c][0] *= corr[hh];
+        acc[hh][c][1] *= corr[hh];
+      }
+    // weighted sum: lane = dims 2 lane, 2 lane + 1 (+ 128 per pass); dim is even (dim % VEC == 0)
     for (int jj = 0; jj < n; ++jj) {
       const f32x4 pv = *reinterpret_cast<const f32x4*>(pw + jj * kHeadChunk);
+      const float ph[kHeadChunk] = {pv.x, pv.y, pv.z, pv.w};
 #pragma unroll
-      for (int c = 0; c < kAccum; ++c) {
-        const int d = lane + c * kWave;
+      for (int c = 0; c < kPairs; ++c) {
+        const int d = 2 * lane + c * 2 * kWave;
         if (d < dim) {
-          const float kv = S::to_f32(tile[(size_t)jj * row_len + d]);
+          float k0, k1;
+          if constexpr (sizeof(T) == 4) {
+            const f32x2 kk = *reinterpret_cast<const f32x2*>(tile + (size_t)jj * row_len + d);
+            k0 = kk.x;
+            k1 = kk.y;
+          } else {
+            const uint32_t kk = *reinterpret_cast<const uint32_t*>(tile + (size_t)jj * row_len + d);
+            k0 = lo16<S>(kk);
+            k1 = hi16<S>(kk);
+          }
 #pragma unroll
-          for (int hh = 0; hh < kHeadChunk; ++hh) acc[hh][c] += pv[hh] * kv;
+          for (int hh = 0; hh < kHeadChunk; ++hh) {
+            acc[hh][c][0] += ph[hh] * k0;
+            acc[hh][c][1] += ph[hh] * k1;
+          }
         }
       }
     }
@@ -252,9 +283,12 @@ __global__ __launch_bounds__(256) void window_attention_group_kernel(
       mine[hh * (2 + dim) + 1] = l[hh];
     }
 #pragma unroll
-    for (int c = 0; c < kAccum; ++c) {
-      const int d = lane + c * kWave;
-      if (d < dim) mine[hh * (2 + dim) + 2 + d] = acc[hh][c];
+    for (int c = 0; c < kPairs; ++c) {
+      const int d = 2 * lane + c * 2 * kWave;
+      if (d < dim) {
+        mine[hh * (2 + dim) + 2 + d] = acc[hh][c][0];
+        mine[hh * (2 + dim) + 2 + d + 1] = acc[hh][c][1];
+      }
     }
   }
   __syncthreads();
@@ -277,7 +311,6 @@ __global__ __launch_bounds__(256) void window_attention_group_kernel(
     out[(int64_t)t * out_stride + (int64_t)(h0 + hh) * dim + d] = S::from_f32(v);
   }
 }
-
 
 // ---------------------------------------------------------------------------------------------
 // window_attention_tile_kernel<S, DB>: prompts and portions of prompts in 16-bit models, on the
@@ -539,8 +572,7 @@ extern "C" int vla_seq_window_attention(void* out, int64_t out_stride, const voi
     // the grouped kernel wants 16-byte rows everywhere it loads vectors and its tiles in LDS
     const int row_pad = VEC;
     const size_t lds = (size_t)4 * kWave * (dim + row_pad) * sizeof(T) +
-                       sizeof(float) * ((size_t)kHeadChunk * dim + 4 * kWave * kHeadChunk +
-                                        (size_t)4 * kHeadChunk * (2 + dim));
+                       sizeof(float) * ((size_t)4 * kWave * kHeadChunk + (size_t)4 * kHeadChunk * (2 + dim));
     const bool grouped = g_window_kernel.load(std::memory_order_relaxed) != 1 && dim % VEC == 0 &&
                          ((uintptr_t)cache % 16) == 0 && lds <= 150 * 1024;
     if (grouped) {
