@@ -122,8 +122,9 @@ class PagedKeys:
 
     def attend(self, q, k, gate, lo, hi, H, window, scale, slopes, coef=0.0, every=1.0, out_scale=1.0,
                kernel="auto"):
-        """kernel: "auto" (rows, picked per shape), "simple" (one wave per row and head), "tiles"
-        (matrix cores, 16-bit only)."""
+        """kernel: "auto" (rows, picked per shape: matrix cores for 16-bit rows), "grouped" (rows, no
+        matrix cores), "simple" (one wave per row and head), "tiles" (runs of rows on the matrix
+        cores, 16-bit only)."""
         n = hi - lo
         pos = torch.arange(lo, hi)
         slots = (self.table[pos // self.bs].long() * self.bs + pos % self.bs).to(DEV)
@@ -136,7 +137,7 @@ class PagedKeys:
                                          self.cache, self.table[None].contiguous().to(DEV), i32([0, n]), i32([lo]), n,
                                          sl, H, window, scale, coef, every, out_scale)
             return out.cpu()
-        ops().set_window_kernel(1 if kernel == "simple" else 0)
+        ops().set_window_kernel({"simple": 1, "grouped": 2}.get(kernel, 0))
         try:
             self._rows(out, q, gate, lo, hi, pos, sl, H, window, scale, coef, every, out_scale)
         finally:
@@ -206,12 +207,14 @@ def test_window_attention_tiles(H, G, D, window, bs, n, dtype):
     want = R.windowed_key_attention(q.to(R.F), k.to(R.F), torch.arange(n), H, G, D, window, scale, coef, every, slopes)
     want = want * torch.sigmoid(gate.to(R.F)) * 0.6
     ulp = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
-    for sizes in ([n], [5, 33, 2, 40, 31, 32, 64]):
+    # whole, portions (tiles), single rows on the matrix cores (auto) and off them (grouped)
+    for sizes, kernel in (([n], "tiles"), ([5, 33, 2, 40, 31, 32, 64], "tiles"), ([1], "auto"), ([1], "grouped"),
+                          ([7, 1, 1], "auto")):
         pk = PagedKeys(G, D, bs, n, dtype=dtype, seed=len(sizes))
         got, lo, i = [], 0, 0
         while lo < n:
             step = min(sizes[i % len(sizes)], n - lo)
-            got.append(pk.attend(q, k, gate, lo, lo + step, H, window, scale, slopes, coef, every, 0.6, "tiles"))
+            got.append(pk.attend(q, k, gate, lo, lo + step, H, window, scale, slopes, coef, every, 0.6, kernel))
             lo += step
             i += 1
         close(torch.cat(got).float(), want, 1.5 * ulp)
@@ -249,6 +252,13 @@ def test_window_attention_tiles_batch_matches_rows():
                                  D**-0.5, 0.3, 16.0)
     ops().window_attention(b_, q, None, cache, bt.to(DEV), tseq, pos, slopes, H, window, D**-0.5, 0.3, 16.0)
     close(a.float(), b_.cpu().float(), 2.0**-7)
+    c_ = torch.empty_like(q)
+    ops().set_window_kernel(2)
+    try:
+        ops().window_attention(c_, q, None, cache, bt.to(DEV), tseq, pos, slopes, H, window, D**-0.5, 0.3, 16.0)
+    finally:
+        ops().set_window_kernel(0)
+    close(b_.float(), c_.cpu().float(), 2.0**-7)
 
 
 def test_window_attention_without_bias_temperature_or_gate_in_bf16():
@@ -262,13 +272,13 @@ def test_window_attention_without_bias_temperature_or_gate_in_bf16():
 
 
 @pytest.mark.parametrize("window,bs", [(5, 4), (16, 16), (17, 16), (32, 16), (33, 8), (64, 16), (65, 8), (100, 32)])
-@pytest.mark.parametrize("decode", [False, True, "tiles"])
+@pytest.mark.parametrize("decode", [False, True, "tiles", "heads"])
 def test_window_edge_decides_the_result(window, bs, decode):
     """Query i and key j share a long vector.  j = i - window + 1 is the last key inside: the
     result is that key.  j = i - window is the first outside: the result is far from it.  i is
     placed so that j falls on the first slot of a page, the last slot of a page, and position 0."""
     H, G, D = 2, 1, 32
-    dt = torch.bfloat16 if decode == "tiles" else torch.float32
+    dt = torch.bfloat16 if decode in ("tiles", "heads") else torch.float32
     n = 3 * window + 2 * bs + 3
     scale = D**-0.5
     for inside in (True, False):
@@ -290,6 +300,10 @@ def test_window_edge_decides_the_result(window, bs, decode):
                 pk.attend(q, k, None, 0, cut, H, window, scale, R.head_slopes(H), kernel="tiles")
                 out = pk.attend(q, k, None, cut, n, H, window, scale, R.head_slopes(H), kernel="tiles")[i - cut].float()
                 k = k.float()
+            elif decode == "heads":         # 16-bit single rows: the matrix-core row kernel
+                pk.attend(q, k, None, 0, i, H, window, scale, R.head_slopes(H), kernel="tiles")
+                out = pk.attend(q, k, None, i, i + 1, H, window, scale, R.head_slopes(H))[0].float()
+                k = k.float()
             elif decode:
                 pk.attend(q, k, None, 0, i, H, window, scale, R.head_slopes(H))
                 out = pk.attend(q, k, None, i, i + 1, H, window, scale, R.head_slopes(H))[0]
@@ -297,7 +311,7 @@ def test_window_edge_decides_the_result(window, bs, decode):
                 out = pk.attend(q, k, None, 0, n, H, window, scale, R.head_slopes(H))[i]
             for h in range(H):
                 d = float((out[h * D:(h + 1) * D] - k[j]).norm() / k[j].norm())
-                assert (d < (1e-2 if decode == "tiles" else 1e-3)) if inside else (d > 0.5), (inside, i, j, h, d)
+                assert (d < (1e-2 if decode in ("tiles", "heads") else 1e-3)) if inside else (d > 0.5), (inside, i, j, h, d)
 
 
 def test_query_temperature_steps_at_multiples_of_its_period():

@@ -8,6 +8,7 @@ parameter is a constructor argument; `None` / 0 switch a term off.  Prompts, por
 and decode steps take the same kernel (csrc/seq_window_attention.hip) after the step's keys have
 been written to the cache.
 """
+import os
 from typing import List, Optional, Tuple
 
 import torch
@@ -24,7 +25,7 @@ def geometric_slopes(num_heads: int, span: float = 8.0) -> List[float]:
 
 class WindowedKeyAttention(nn.Module):
     # steps whose longest run of rows is at least this long take the tiled kernel (16-bit models)
-    TILE_MIN_QUERY = 4
+    TILE_MIN_QUERY = int(os.environ.get("VLA_TILE_MIN_QUERY", "4"))
 
     def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, scale: float,
                  window: Optional[int] = None, slopes: Optional[List[float]] = None,

@@ -14,6 +14,7 @@
 // The state is read from its slot unless the sequence starts here (context length 0), and
 // written back at the end: a slot needs no clearing before it is used again.
 #include <atomic>
+#include <cstdlib>
 
 #include "seq_common.h"
 
@@ -22,6 +23,11 @@ namespace seq {
 namespace {
 
 std::atomic<int> g_scan_kernel{0};
+std::atomic<int> g_scan_cols{[] {
+  const char* e = getenv("VLA_SCAN_COLS");
+  const int v = e ? atoi(e) : 16;
+  return v >= 1 && v <= 256 ? v : 16;
+}()};
 
 template <class S>
 __global__ __launch_bounds__(256) void gla_log_decay_kernel(
@@ -294,9 +300,10 @@ extern "C" int vla_seq_gla_scan(float* o, const void* q, int64_t q_stride, const
       q_stride < (int64_t)heads * dim || k_stride < (int64_t)heads * dim ||
       v_stride < (int64_t)heads * vdim)
     return VLA_ERR_ARG;
-  // ---- the blocked walk: slices of at most 64 value columns, up to 256 threads
+  // ---- the blocked walk: slices of at most kSliceCols value columns, up to 256 threads
   {
-    const int vb = vdim < 64 ? vdim : 64;
+    const int cols = g_scan_cols.load(std::memory_order_relaxed);
+    const int vb = vdim < cols ? vdim : cols;
     const int slices = (vdim + vb - 1) / vb;
     int groups = 256 / vb;
     if (groups > dim) groups = dim;

@@ -500,6 +500,228 @@ __global__ __launch_bounds__(256) void window_attention_tile_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// window_attention_heads_kernel<S, DB>: single rows (decode steps) of 16-bit models on the matrix
+// cores.  One workgroup per (row, KV head, chunk of up to 32 of its query heads).  The products
+// are those of the tile kernel with the 32 columns holding the chunk's query heads instead of 32
+// rows of one head: S^T = K q^T scores one 32-key tile against every head at once, so each key
+// byte is read once per KV head whatever the group size.  The four waves split the window's
+// tiles (wave w takes tiles w, w + 4, ...), each with its own tile in LDS and its own running
+// max / sum / output, merged at the end.
+template <class S, int DB>
+__global__ __launch_bounds__(256) void window_attention_heads_kernel(
+    typename S::T* __restrict__ out, int64_t out_stride, const typename S::T* __restrict__ q,
+    int64_t q_stride, const typename S::T* __restrict__ gate, int64_t gate_stride,
+    const typename S::T* __restrict__ cache, const int* __restrict__ block_tables, int max_blocks,
+    const int* __restrict__ token_seq, const int64_t* __restrict__ positions,
+    const float* __restrict__ slopes, int heads, int kv_heads, int block_size, int num_blocks,
+    int window, float scale, float temp_coef, float temp_every, float out_scale) {
+  using T = typename S::T;
+  using M = Mfma8<S>;
+  constexpr int D = 32 * DB;
+  constexpr int KROW = D + 4, TROW = kTile + 4;
+  constexpr int WAVE_ELEMS = kTile * KROW + D * TROW;     // one wave's two tiles, in elements
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int hf = lane >> 5, c = lane & 31;
+  T* k_lds = reinterpret_cast<T*>(smem) + (size_t)w * WAVE_ELEMS;
+  T* kt_lds = k_lds + kTile * KROW;
+  const int t = blockIdx.x;
+  const int group = heads / kv_heads;
+  const int chunks = (group + 31) / 32;
+  const int g = blockIdx.y / chunks;
+  const int h0 = g * group + (blockIdx.y % chunks) * 32;
+  const int nh = min(32, g * group + group - h0);
+  const int p = (int)positions[t];
+  const int* table = block_tables + (int64_t)token_seq[t] * max_blocks;
+  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int64_t tok_stride = (int64_t)kv_heads * D;
+  float qs = scale;
+  if (temp_coef != 0.f) qs *= 1.f + temp_coef * logf(floorf((float)(p + 1) / temp_every) + 1.f);
+  const bool live = c < nh;
+  const float slope = (slopes != nullptr && live) ? slopes[h0 + c] : 0.f;
+  u32x2 qf[D / 8];
+#pragma unroll
+  for (int ks = 0; ks < D / 8; ++ks) {
+    u32x2 v = {0u, 0u};
+    if (live)
+      v = *reinterpret_cast<const u32x2*>(q + (int64_t)t * q_stride + (int64_t)(h0 + c) * D + 8 * ks + 4 * hf);
+    qf[ks] = v;
+  }
+  f32x16 o[DB];
+#pragma unroll
+  for (int n = 0; n < DB; ++n)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[n][i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  // A wave's share of a tile is D / 8 pieces of 8 bytes per lane.  Their loads are all issued
+  // before any is used, and one tile ahead: while a tile is in the matrix cores the next one is
+  // on its way from HBM.  (A piece's address needs the key's block from the table: lanes 0..31
+  // look the 32 keys of the tile up once and hand the row offsets round with shuffles.)
+  constexpr int PIECES = D / 8;
+  u32x2 x[PIECES];
+  auto fetch = [&](int j0) {
+    const int jr = j0 + c;
+    long long base = -1;
+    if (jr <= p) {
+      int blk = table[jr / block_size];
+      blk = (unsigned)blk < (unsigned)num_blocks ? blk : 0;
+      base = ((long long)blk * block_size + jr % block_size) * tok_stride + (long long)g * D;
+    }
+#pragma unroll
+    for (int u = 0; u < PIECES; ++u) {
+      const int i = lane + kWave * u;
+      const int r = i / (D / 4), v = i % (D / 4);
+      const long long rb = __shfl(base, r, 64);
+      const T* src = cache + (rb >= 0 ? rb + 4 * v : 0);     // a valid address either way
+      const u32x2 got = *reinterpret_cast<const u32x2*>(src);
+      x[u] = rb >= 0 ? got : u32x2{0u, 0u};
+    }
+  };
+  fetch(lo + w * kTile);
+  for (int j0 = lo + w * kTile; j0 <= p; j0 += 4 * kTile) {
+#pragma unroll
+    for (int u = 0; u < PIECES; ++u) {
+      const int i = lane + kWave * u;
+      const int r = i / (D / 4), v = i % (D / 4);
+      *reinterpret_cast<u32x2*>(k_lds + r * KROW + 4 * v) = x[u];
+      uint16_t* col = reinterpret_cast<uint16_t*>(kt_lds) + (4 * v) * TROW + r;
+      col[0] = (uint16_t)(x[u][0] & 0xffffu);
+      col[TROW] = (uint16_t)(x[u][0] >> 16);
+      col[2 * TROW] = (uint16_t)(x[u][1] & 0xffffu);
+      col[3 * TROW] = (uint16_t)(x[u][1] >> 16);
+    }
+    if (j0 + 4 * kTile <= p) fetch(j0 + 4 * kTile);
+    wave_sync();
+    f32x16 st;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) st[i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < D / 8; ++ks) {
+      const u32x2 a = *reinterpret_cast<const u32x2*>(k_lds + c * KROW + 8 * ks + 4 * hf);
+      st = M::run(a, qf[ks], st);
+    }
+    float mt = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int dist = p - (j0 + (i & 3) + 8 * (i >> 2) + 4 * hf);
+      st[i] = (live && dist >= 0) ? st[i] * qs - slope * (float)dist : -INFINITY;
+      mt = fmaxf(mt, st[i]);
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(m, mt);
+    const float corr = m_new == -INFINITY ? 1.f : expf(m - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      st[i] = m_new == -INFINITY ? 0.f : expf(st[i] - m_new);
+      psum += st[i];
+    }
+    l = l * corr + psum;
+    m = m_new;
+#pragma unroll
+    for (int n = 0; n < DB; ++n)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[n][i] *= corr;
+#pragma unroll
+    for (int s8 = 0; s8 < 4; ++s8) {
+      uint32_t hb[4], lb[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float pv = st[4 * s8 + e];
+        hb[e] = bits16<S>(pv);
+        lb[e] = bits16<S>(pv - from_bits16<S>(hb[e]));
+      }
+      const u32x2 hi = {hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16)};
+      const u32x2 lo2 = {lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16)};
+#pragma unroll
+      for (int n = 0; n < DB; ++n) {
+        const u32x2 a = *reinterpret_cast<const u32x2*>(kt_lds + (32 * n + c) * TROW + 8 * s8 + 4 * hf);
+        o[n] = M::run(a, hi, o[n]);
+        o[n] = M::run(a, lo2, o[n]);
+      }
+    }
+    wave_sync();
+  }
+  l += __shfl_xor(l, 32, 64);
+  // merge the four waves through LDS (the tiles are done with): [wave][head][2 + D]
+  __syncthreads();
+  float* merge = reinterpret_cast<float*>(smem);
+  if (live) {
+    float* mine = merge + ((size_t)w * 32 + c) * (2 + D);
+    if (hf == 0) {
+      mine[0] = m;
+      mine[1] = l;
+    }
+#pragma unroll
+    for (int n = 0; n < DB; ++n)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mine[2 + 32 * n + (i & 3) + 8 * (i >> 2) + 4 * hf] = o[n][i];
+  }
+  __syncthreads();
+  for (int i = tid; i < nh * D; i += 256) {
+    const int hh = i / D, d = i - hh * D;
+    float mm = -INFINITY;
+    for (int ww = 0; ww < 4; ++ww) mm = fmaxf(mm, merge[((size_t)ww * 32 + hh) * (2 + D)]);
+    float ll = 0.f, ov = 0.f;
+    for (int ww = 0; ww < 4; ++ww) {
+      const float* src = merge + ((size_t)ww * 32 + hh) * (2 + D);
+      const float f = src[0] == -INFINITY ? 0.f : expf(src[0] - mm);
+      ll += src[1] * f;
+      ov += src[2 + d] * f;
+    }
+    float v = ov * (out_scale / ll);
+    if (gate != nullptr) {
+      const float gv = S::to_f32(gate[(int64_t)t * gate_stride + (int64_t)(h0 + hh) * D + d]);
+      v *= 1.f / (1.f + expf(-gv));
+    }
+    out[(int64_t)t * out_stride + (int64_t)(h0 + hh) * D + d] = S::from_f32(v);
+  }
+}
+
+template <class S, int DB>
+size_t heads_kernel_lds() {
+  constexpr int D = 32 * DB;
+  const size_t tiles = (size_t)4 * (kTile * (D + 4) + D * (kTile + 4)) * sizeof(typename S::T);
+  const size_t merge = (size_t)4 * 32 * (2 + D) * sizeof(float);
+  return tiles > merge ? tiles : merge;
+}
+
+template <class S, int DB>
+int launch_heads_one(dim3 grid, hipStream_t stream, typename S::T* out, int64_t out_stride,
+                     const typename S::T* q, int64_t q_stride, const typename S::T* gate,
+                     int64_t gate_stride, const typename S::T* cache, const int* block_tables,
+                     int max_blocks, const int* token_seq, const int64_t* positions,
+                     const float* slopes, int heads, int kv_heads, int block_size, int num_blocks,
+                     int window, float scale, float temp_coef, float temp_every, float out_scale) {
+  const size_t lds = heads_kernel_lds<S, DB>();
+  static std::atomic<size_t> allowed{64 * 1024};   // raised once per kernel, not per launch
+  if (lds > allowed.load(std::memory_order_relaxed)) {
+    VLA_SEQ_HIP_CHECK(hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&window_attention_heads_kernel<S, DB>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    allowed.store(lds, std::memory_order_relaxed);
+  }
+  window_attention_heads_kernel<S, DB><<<grid, 256, lds, stream>>>(
+      out, out_stride, q, q_stride, gate, gate_stride, cache, block_tables, max_blocks, token_seq,
+      positions, slopes, heads, kv_heads, block_size, num_blocks, window, scale, temp_coef,
+      temp_every, out_scale);
+  VLA_SEQ_HIP_CHECK(hipGetLastError());
+  return VLA_OK;
+}
+
+template <class S, class... A>
+int launch_heads(int db, A... a) {
+  switch (db) {
+    case 1: return launch_heads_one<S, 1>(a...);
+    case 2: return launch_heads_one<S, 2>(a...);
+    case 3: return launch_heads_one<S, 3>(a...);
+    case 4: return launch_heads_one<S, 4>(a...);
+    default: return VLA_ERR_HEAD_SIZE;
+  }
+}
+
 template <class S>
 int launch_tiles(int db, dim3 grid, hipStream_t stream, typename S::T* out, int64_t out_stride,
                  const typename S::T* q, int64_t q_stride, const typename S::T* gate,
@@ -573,15 +795,31 @@ extern "C" int vla_seq_window_attention(void* out, int64_t out_stride, const voi
     const int row_pad = VEC;
     const size_t lds = (size_t)4 * kWave * (dim + row_pad) * sizeof(T) +
                        sizeof(float) * ((size_t)4 * kWave * kHeadChunk + (size_t)4 * kHeadChunk * (2 + dim));
-    const bool grouped = g_window_kernel.load(std::memory_order_relaxed) != 1 && dim % VEC == 0 &&
+    const int mode = g_window_kernel.load(std::memory_order_relaxed);
+    if constexpr (sizeof(T) == 2) {
+      // 16-bit rows on the matrix cores when the head size and the alignment allow
+      if (mode == 0 && dim % 32 == 0 && dim <= 128 && ((uintptr_t)q % 8) == 0 &&
+          ((q_stride * 2) % 8) == 0 && ((uintptr_t)cache % 8) == 0) {
+        const int group = heads / kv_heads;
+        const dim3 grid(num_tokens, kv_heads * ((group + 31) / 32));
+        return launch_heads<S>(dim / 32, grid, (hipStream_t)stream, (T*)out, out_stride, (const T*)q,
+                               q_stride, (const T*)gate, gate_stride, (const T*)cache, block_tables,
+                               max_blocks, token_seq, positions, slopes, heads, kv_heads, block_size,
+                               num_blocks, window, scale, temp_coef, temp_every, out_scale);
+      }
+    }
+    const bool grouped = mode != 1 && dim % VEC == 0 &&
                          ((uintptr_t)cache % 16) == 0 && lds <= 150 * 1024;
     if (grouped) {
       const int group = heads / kv_heads;
       const dim3 grid(num_tokens, kv_heads * ((group + kHeadChunk - 1) / kHeadChunk));
-      if (lds > 64 * 1024)
+      static std::atomic<size_t> allowed{64 * 1024};   // raised once per kernel, not per launch
+      if (lds > allowed.load(std::memory_order_relaxed)) {
         VLA_SEQ_HIP_CHECK(hipFuncSetAttribute(
             reinterpret_cast<const void*>(&window_attention_group_kernel<S>),
             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        allowed.store(lds, std::memory_order_relaxed);
+      }
       window_attention_group_kernel<S><<<grid, 256, lds, (hipStream_t)stream>>>(
           (T*)out, out_stride, (const T*)q, q_stride, (const T*)gate, gate_stride, (const T*)cache,
           block_tables, max_blocks, token_seq, positions, slopes, heads, kv_heads, dim, block_size,
@@ -599,7 +837,8 @@ extern "C" int vla_seq_window_attention(void* out, int64_t out_stride, const voi
   });
 }
 
-// 0: pick per shape; 1: the one-wave-per-(row, head) kernel; (tests run both)
+// 0: pick per shape; 1: the one-wave-per-(row, head) kernel; 2: no matrix-core kernel for rows
+// (tests run all)
 extern "C" int vla_seq_set_window_kernel(int mode) {
   if (mode < 0 || mode > 2) return VLA_ERR_ARG;
   g_window_kernel.store(mode, std::memory_order_relaxed);
