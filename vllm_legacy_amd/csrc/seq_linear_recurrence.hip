@@ -25,8 +25,8 @@ namespace {
 std::atomic<int> g_scan_kernel{0};
 std::atomic<int> g_scan_cols{[] {
   const char* e = getenv("VLA_SCAN_COLS");
-  const int v = e ? atoi(e) : 16;
-  return v >= 1 && v <= 256 ? v : 16;
+  const int v = e ? atoi(e) : 0;     // 0: by the step's longest run of rows
+  return v >= 0 && v <= 256 ? v : 0;
 }()};
 
 template <class S>
@@ -160,27 +160,35 @@ __global__ __launch_bounds__(256) void gla_scan_block_kernel(
     const int d = row0 + i;
     s[i] = (owner && d < dim && context_lens[b] > 0) ? sp[(int64_t)d * vdim + col] : 0.f;
   }
-  float regs[kStageLoads];
+  float regs_a[kStageLoads], regs_b[kStageLoads];   // blocks in flight: odd ones in a, even in b
   const int tt_step = nthreads / tok, e_step = nthreads - tt_step * tok;
   // global -> registers.  Every thread issues all its loads before it needs any of them: the
   // addresses of entries that do not exist (padding, tokens past the block) are bent to a row that
   // does, and the value is dropped afterwards, so no load sits behind a branch.
-  auto fetch = [&](int tstart, int n) {
+  auto fetch = [&](int tstart, int n, float (&regs)[kStageLoads]) {
     int tt = tid / tok, e = tid - tt * tok;      // element tid + u * nthreads = (token tt, entry e)
-    const T* safe_t = q + (int64_t)tstart * q_stride + (int64_t)h * dim;
-    const float* safe_f = log_decay + ((int64_t)tstart * heads + h) * dim;
+    // row bases of the block's first token are wave-uniform (scalar arithmetic); what a lane adds
+    // is a 32-bit offset from a 24-bit multiply (strides below 2^24 are a launch condition):
+    // 64-bit per-lane multiplies here cost more than the walk itself
+    const T* qb = q + (int64_t)tstart * q_stride + (int64_t)h * dim;
+    const T* kb = k + (int64_t)tstart * k_stride + (int64_t)h * dim;
+    const T* vbase = v + (int64_t)tstart * v_stride + (int64_t)h * vdim + v0;
+    const float* db = log_decay + ((int64_t)tstart * heads + h) * dim;
+    const T* safe_t = qb;
+    const float* safe_f = db;
+    const unsigned qs32 = (unsigned)q_stride, ks32 = (unsigned)k_stride, vs32 = (unsigned)v_stride,
+                   ds32 = (unsigned)(heads * dim);
     float xt[kStageLoads], xf[kStageLoads];
     int kind[kStageLoads];                       // 0 q, 1 k, 2 decay, 3 v, -1 nothing
 #pragma unroll
     for (int u = 0; u < kStageLoads; ++u) {
-      const int64_t t = tstart + tt;
       const int sec = e < dim_pad ? 0 : (e < 2 * dim_pad ? 1 : (e < 3 * dim_pad ? 2 : 3));
       const int off = e - sec * dim_pad;
       const bool valid = tt < n && (sec < 3 ? off < dim : off < nv);
-      const T* pt = sec == 0 ? q + t * q_stride + (int64_t)h * dim + off
-                             : (sec == 1 ? k + t * k_stride + (int64_t)h * dim + off
-                                         : v + t * v_stride + (int64_t)h * vdim + v0 + off);
-      const float* pf = log_decay + (t * heads + h) * dim + off;
+      const unsigned ut = (unsigned)tt;
+      const T* pt = sec == 0 ? qb + (__umul24(ut, qs32) + off)
+                             : (sec == 1 ? kb + (__umul24(ut, ks32) + off) : vbase + (__umul24(ut, vs32) + off));
+      const float* pf = db + (__umul24(ut, ds32) + off);
       pt = (valid && sec != 2) ? pt : safe_t;
       pf = (valid && sec == 2) ? pf : safe_f;
       xt[u] = S::to_f32(*pt);
@@ -199,52 +207,82 @@ __global__ __launch_bounds__(256) void gla_scan_block_kernel(
       regs[u] = kind[u] < 0 ? 0.f : x;
     }
   };
-  auto put = [&](float* buf, int n) {            // registers -> LDS
+  auto put = [&](float* buf, int n, const float (&regs)[kStageLoads]) {   // registers -> LDS
 #pragma unroll
     for (int u = 0; u < kStageLoads; ++u) {
       const int i = tid + u * nthreads;
       if (i < n * tok) buf[i] = regs[u];
     }
   };
-  fetch(t0, min(tb, t1 - t0));
-  put(lds, min(tb, t1 - t0));
+  // Block i is staged in LDS buffer i & 1 while block i + 1 is on its way in one register set and
+  // the loads of block i + 2 are issued into the other: a block's loads have a whole iteration
+  // before anyone waits for them.
+  fetch(t0, min(tb, t1 - t0), regs_b);
+  put(lds, min(tb, t1 - t0), regs_b);
+  if (t0 + tb < t1) fetch(t0 + tb, min(tb, t1 - (t0 + tb)), regs_a);
   __syncthreads();
-  int parity = 0;
-  for (int ts = t0; ts < t1; ts += tb, parity ^= 1) {
+  auto iteration = [&](int ts, int parity, float (&arriving)[kStageLoads], float (&issue)[kStageLoads]) {
     const int n = min(tb, t1 - ts);
     const int nn = min(tb, t1 - (ts + tb));          // next block's tokens (<= 0: none)
+    const int n2 = min(tb, t1 - (ts + 2 * tb));      // the one after
     float* cur = lds + parity * per;
     float* part = cur + tb * tok;
-    if (nn > 0) fetch(ts + tb, nn);
     if (owner) {
-      for (int tt = 0; tt < n; ++tt) {
-        const float* in = cur + tt * tok;
-        const float vv = in[3 * dim_pad + col];
-        float acc = 0.f;
-        if constexpr (ROWS % 4 == 0) {
+      if constexpr (ROWS % 4 == 0) {
+        // TU tokens at a time: all their LDS reads first, then the walk, then the partial sums --
+        // a read of the next token cannot wait behind the write of the previous one's sum.  Rows
+        // of the stage past the block's tokens hold old values: they are read and not used.
+        constexpr int TU = ROWS <= 4 ? 4 : (ROWS <= 8 ? 2 : 1);
+        for (int tt = 0; tt < n; tt += TU) {
+          f32x4 q4[TU][ROWS / 4], k4[TU][ROWS / 4], a4[TU][ROWS / 4];
+          float vv[TU], acc[TU];
 #pragma unroll
-          for (int i = 0; i < ROWS; i += 4) {
-            const f32x4 q4 = *reinterpret_cast<const f32x4*>(in + row0 + i);
-            const f32x4 k4 = *reinterpret_cast<const f32x4*>(in + dim_pad + row0 + i);
-            const f32x4 a4 = *reinterpret_cast<const f32x4*>(in + 2 * dim_pad + row0 + i);
-            s[i] = a4.x * s[i] + k4.x * vv;
-            s[i + 1] = a4.y * s[i + 1] + k4.y * vv;
-            s[i + 2] = a4.z * s[i + 2] + k4.z * vv;
-            s[i + 3] = a4.w * s[i + 3] + k4.w * vv;
-            acc += s[i] * q4.x + s[i + 1] * q4.y + s[i + 2] * q4.z + s[i + 3] * q4.w;
+          for (int u = 0; u < TU; ++u) {
+            const float* in = cur + min(tt + u, tb - 1) * tok;
+            vv[u] = in[3 * dim_pad + col];
+#pragma unroll
+            for (int i = 0; i < ROWS / 4; ++i) {
+              q4[u][i] = *reinterpret_cast<const f32x4*>(in + row0 + 4 * i);
+              k4[u][i] = *reinterpret_cast<const f32x4*>(in + dim_pad + row0 + 4 * i);
+              a4[u][i] = *reinterpret_cast<const f32x4*>(in + 2 * dim_pad + row0 + 4 * i);
+            }
           }
-        } else {
+#pragma unroll
+          for (int u = 0; u < TU; ++u) {
+            acc[u] = 0.f;
+            if (tt + u < n) {
+#pragma unroll
+              for (int i = 0; i < ROWS / 4; ++i) {
+                s[4 * i] = a4[u][i].x * s[4 * i] + k4[u][i].x * vv[u];
+                s[4 * i + 1] = a4[u][i].y * s[4 * i + 1] + k4[u][i].y * vv[u];
+                s[4 * i + 2] = a4[u][i].z * s[4 * i + 2] + k4[u][i].z * vv[u];
+                s[4 * i + 3] = a4[u][i].w * s[4 * i + 3] + k4[u][i].w * vv[u];
+                acc[u] += s[4 * i] * q4[u][i].x + s[4 * i + 1] * q4[u][i].y + s[4 * i + 2] * q4[u][i].z +
+                          s[4 * i + 3] * q4[u][i].w;
+              }
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < TU; ++u)
+            if (tt + u < n) part[((tt + u) * groups + grp) * vb + col] = acc[u];
+        }
+      } else {
+        for (int tt = 0; tt < n; ++tt) {
+          const float* in = cur + tt * tok;
+          const float vv = in[3 * dim_pad + col];
+          float acc = 0.f;
 #pragma unroll
           for (int i = 0; i < ROWS; ++i) {
             const int d = row0 + i;
             s[i] = in[2 * dim_pad + d] * s[i] + in[dim_pad + d] * vv;
             acc += s[i] * in[d];
           }
+          part[(tt * groups + grp) * vb + col] = acc;
         }
-        part[(tt * groups + grp) * vb + col] = acc;
       }
     }
-    if (nn > 0) put(lds + (parity ^ 1) * per, nn);
+    if (nn > 0) put(lds + (parity ^ 1) * per, nn, arriving);
+    if (n2 > 0) fetch(ts + 2 * tb, n2, issue);       // `issue` held this block: free since its put
     __syncthreads();
     for (int i = tid; i < n * vb; i += nthreads) {
       const int tt = i / vb, c = i - tt * vb;
@@ -254,6 +292,10 @@ __global__ __launch_bounds__(256) void gla_scan_block_kernel(
         o[((int64_t)(ts + tt) * heads + h) * vdim + v0 + c] = sum;
       }
     }
+  };
+  for (int ts = t0; ts < t1; ts += 2 * tb) {
+    iteration(ts, 0, regs_a, regs_b);
+    if (ts + tb < t1) iteration(ts + tb, 1, regs_b, regs_a);
   }
   if (owner) {
 #pragma unroll
@@ -302,7 +344,13 @@ extern "C" int vla_seq_gla_scan(float* o, const void* q, int64_t q_stride, const
     return VLA_ERR_ARG;
   // ---- the blocked walk: slices of at most kSliceCols value columns, up to 256 threads
   {
-    const int cols = g_scan_cols.load(std::memory_order_relaxed);
+    // Slice width: a walk of many tokens is bound by its serial chain, so narrow slices (more
+    // workgroups, fewer rows per thread) win; a walk of a token or two is bound by reading and
+    // writing the state, which wide slices do in fewer, fuller workgroups.  Measured on
+    // 16 heads x 64 x 128: 4096 tokens 1.45 ms at 16 columns against 2.03 ms at 64; 64 sequences
+    // of one token 40 us at 64 columns against 120 us at 16.
+    int cols = g_scan_cols.load(std::memory_order_relaxed);
+    if (cols == 0) cols = (max_query_len > 0 && max_query_len <= 4) ? 64 : 16;
     const int vb = vdim < cols ? vdim : cols;
     const int slices = (vdim + vb - 1) / vb;
     int groups = 256 / vb;
@@ -318,13 +366,28 @@ extern "C" int vla_seq_gla_scan(float* o, const void* q, int64_t q_stride, const
     if (max_query_len > 0 && tb > max_query_len) tb = max_query_len;   // decode: small LDS, many workgroups
     const int per = tb * tok + ((tb * groups * vb + 3) & ~3);
     const size_t lds_bytes = 2 * (size_t)per * sizeof(float);
-    if (g_scan_kernel.load(std::memory_order_relaxed) != 1 && rows_pow2 <= 64 && tb >= 1 &&
-        lds_bytes <= 64 * 1024) {
+    // a step of single rows has nothing to block: the token-by-token kernel below does it with
+    // less set-up (64 sequences x 16 heads x 64 x 128: 15 us against 40 us)
+    const int64_t lim24 = (int64_t)1 << 24;
+    if (g_scan_kernel.load(std::memory_order_relaxed) != 1 && max_query_len != 1 && rows_pow2 <= 64 &&
+        q_stride < lim24 && k_stride < lim24 && v_stride < lim24 && (int64_t)heads * dim < lim24 &&
+        tb >= 1 && lds_bytes <= 150 * 1024) {
       return with_dtype(dtype, [&](auto s) {
         using S = decltype(s);
         using T = typename S::T;
         const dim3 grid(heads, num_seqs, slices);
+        int status = VLA_OK;
         auto launch = [&](auto kernel) {
+          static std::atomic<size_t> allowed{64 * 1024};   // raised once per kernel, not per launch
+          if (lds_bytes > allowed.load(std::memory_order_relaxed)) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)lds_bytes) != hipSuccess) {
+              status = VLA_ERR_HIP;
+              return;
+            }
+            allowed.store(lds_bytes, std::memory_order_relaxed);
+          }
           kernel<<<grid, threads, lds_bytes, (hipStream_t)stream>>>(
               o, (const T*)q, q_stride, (const T*)k, k_stride, (const T*)v, v_stride, log_decay, state,
               query_start_loc, context_lens, state_slots, q_scale, heads, dim, vdim, vb, groups, tb,
@@ -339,6 +402,7 @@ extern "C" int vla_seq_gla_scan(float* o, const void* q, int64_t q_stride, const
           case 32: launch(gla_scan_block_kernel<S, 32>); break;
           default: launch(gla_scan_block_kernel<S, 64>); break;
         }
+        if (status != VLA_OK) return status;
         VLA_SEQ_HIP_CHECK(hipGetLastError());
         return VLA_OK;
       });

@@ -410,25 +410,39 @@ __global__ __launch_bounds__(256) void window_attention_tile_kernel(
     for (int i = 0; i < 16; ++i) o[n][i] = 0.f;
   float m = -INFINITY, l = 0.f;
 
-  for (int j0 = j_lo; j0 <= p_last; j0 += kTile) {
-    __syncthreads();
-    for (int i = tid; i < kTile * (D / 4); i += 256) {
-      const int r = i / (D / 4), v = i - r * (D / 4);
+  // staging: DB pieces of 8 bytes per thread and tile, loaded one tile ahead (see the heads kernel)
+  u32x2 x[DB];
+  auto fetch = [&](int j0) {
+#pragma unroll
+    for (int u = 0; u < DB; ++u) {
+      const int i = tid + 256 * u;
+      const int r = i / (D / 4), v = i % (D / 4);
       const int j = j0 + r;
-      u32x2 x = {0u, 0u};
+      long long off = 0;
       if (j <= p_last) {
         int blk = table[j / block_size];
         blk = (unsigned)blk < (unsigned)num_blocks ? blk : 0;
-        x = *reinterpret_cast<const u32x2*>(cache + ((int64_t)blk * block_size + j % block_size) * tok_stride +
-                                            (int64_t)g * D + 4 * v);
+        off = ((long long)blk * block_size + j % block_size) * tok_stride + (long long)g * D + 4 * v;
       }
-      *reinterpret_cast<u32x2*>(k_lds + r * KROW + 4 * v) = x;
-      uint16_t* col = reinterpret_cast<uint16_t*>(kt_lds) + (4 * v) * TROW + r;
-      col[0] = (uint16_t)(x[0] & 0xffffu);
-      col[TROW] = (uint16_t)(x[0] >> 16);
-      col[2 * TROW] = (uint16_t)(x[1] & 0xffffu);
-      col[3 * TROW] = (uint16_t)(x[1] >> 16);
+      const u32x2 got = *reinterpret_cast<const u32x2*>(cache + off);
+      x[u] = j <= p_last ? got : u32x2{0u, 0u};
     }
+  };
+  fetch(j_lo);
+  for (int j0 = j_lo; j0 <= p_last; j0 += kTile) {
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < DB; ++u) {
+      const int i = tid + 256 * u;
+      const int r = i / (D / 4), v = i % (D / 4);
+      *reinterpret_cast<u32x2*>(k_lds + r * KROW + 4 * v) = x[u];
+      uint16_t* col = reinterpret_cast<uint16_t*>(kt_lds) + (4 * v) * TROW + r;
+      col[0] = (uint16_t)(x[u][0] & 0xffffu);
+      col[TROW] = (uint16_t)(x[u][0] >> 16);
+      col[2 * TROW] = (uint16_t)(x[u][1] & 0xffffu);
+      col[3 * TROW] = (uint16_t)(x[u][1] >> 16);
+    }
+    if (j0 + kTile <= p_last) fetch(j0 + kTile);
     __syncthreads();
     if (!active) continue;
     f32x16 st;
@@ -506,10 +520,12 @@ __global__ __launch_bounds__(256) void window_attention_tile_kernel(
 // are those of the tile kernel with the 32 columns holding the chunk's query heads instead of 32
 // rows of one head: S^T = K q^T scores one 32-key tile against every head at once, so each key
 // byte is read once per KV head whatever the group size.  The four waves split the window's
-// tiles (wave w takes tiles w, w + 4, ...), each with its own tile in LDS and its own running
+// tiles (wave w of kRowWaves takes tiles w, w + kRowWaves, ...), each with its own tile in LDS and its own running
 // max / sum / output, merged at the end.
+constexpr int kRowWaves = 8;   // waves that split a row's window
+
 template <class S, int DB>
-__global__ __launch_bounds__(256) void window_attention_heads_kernel(
+__global__ __launch_bounds__(64 * kRowWaves) void window_attention_heads_kernel(
     typename S::T* __restrict__ out, int64_t out_stride, const typename S::T* __restrict__ q,
     int64_t q_stride, const typename S::T* __restrict__ gate, int64_t gate_stride,
     const typename S::T* __restrict__ cache, const int* __restrict__ block_tables, int max_blocks,
@@ -580,7 +596,7 @@ __global__ __launch_bounds__(256) void window_attention_heads_kernel(
     }
   };
   fetch(lo + w * kTile);
-  for (int j0 = lo + w * kTile; j0 <= p; j0 += 4 * kTile) {
+  for (int j0 = lo + w * kTile; j0 <= p; j0 += kRowWaves * kTile) {
 #pragma unroll
     for (int u = 0; u < PIECES; ++u) {
       const int i = lane + kWave * u;
@@ -592,7 +608,7 @@ __global__ __launch_bounds__(256) void window_attention_heads_kernel(
       col[2 * TROW] = (uint16_t)(x[u][1] & 0xffffu);
       col[3 * TROW] = (uint16_t)(x[u][1] >> 16);
     }
-    if (j0 + 4 * kTile <= p) fetch(j0 + 4 * kTile);
+    if (j0 + kRowWaves * kTile <= p) fetch(j0 + kRowWaves * kTile);
     wave_sync();
     f32x16 st;
 #pragma unroll
@@ -660,12 +676,12 @@ __global__ __launch_bounds__(256) void window_attention_heads_kernel(
       for (int i = 0; i < 16; ++i) mine[2 + 32 * n + (i & 3) + 8 * (i >> 2) + 4 * hf] = o[n][i];
   }
   __syncthreads();
-  for (int i = tid; i < nh * D; i += 256) {
+  for (int i = tid; i < nh * D; i += 64 * kRowWaves) {
     const int hh = i / D, d = i - hh * D;
     float mm = -INFINITY;
-    for (int ww = 0; ww < 4; ++ww) mm = fmaxf(mm, merge[((size_t)ww * 32 + hh) * (2 + D)]);
+    for (int ww = 0; ww < kRowWaves; ++ww) mm = fmaxf(mm, merge[((size_t)ww * 32 + hh) * (2 + D)]);
     float ll = 0.f, ov = 0.f;
-    for (int ww = 0; ww < 4; ++ww) {
+    for (int ww = 0; ww < kRowWaves; ++ww) {
       const float* src = merge + ((size_t)ww * 32 + hh) * (2 + D);
       const float f = src[0] == -INFINITY ? 0.f : expf(src[0] - mm);
       ll += src[1] * f;
@@ -683,8 +699,8 @@ __global__ __launch_bounds__(256) void window_attention_heads_kernel(
 template <class S, int DB>
 size_t heads_kernel_lds() {
   constexpr int D = 32 * DB;
-  const size_t tiles = (size_t)4 * (kTile * (D + 4) + D * (kTile + 4)) * sizeof(typename S::T);
-  const size_t merge = (size_t)4 * 32 * (2 + D) * sizeof(float);
+  const size_t tiles = (size_t)kRowWaves * (kTile * (D + 4) + D * (kTile + 4)) * sizeof(typename S::T);
+  const size_t merge = (size_t)kRowWaves * 32 * (2 + D) * sizeof(float);
   return tiles > merge ? tiles : merge;
 }
 
@@ -703,7 +719,7 @@ int launch_heads_one(dim3 grid, hipStream_t stream, typename S::T* out, int64_t 
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     allowed.store(lds, std::memory_order_relaxed);
   }
-  window_attention_heads_kernel<S, DB><<<grid, 256, lds, stream>>>(
+  window_attention_heads_kernel<S, DB><<<grid, 64 * kRowWaves, lds, stream>>>(
       out, out_stride, q, q_stride, gate, gate_stride, cache, block_tables, max_blocks, token_seq,
       positions, slopes, heads, kv_heads, block_size, num_blocks, window, scale, temp_coef,
       temp_every, out_scale);
