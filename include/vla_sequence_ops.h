@@ -97,6 +97,21 @@ int vla_seq_gla_scan(float* o, const void* q, int64_t q_stride, const void* k, i
                      float q_scale, int num_seqs, int num_slots, int max_query_len, int heads,
                      int dim, int vdim, int dtype, void* stream);
 
+/* A long run of rows cut into pieces that are walked at once (each from a zero state, through
+ * vla_seq_gla_scan with one entry per piece): with c_t the sum of the log decays from a piece's
+ * first row to row t, vla_seq_gla_piece_prefix writes q_decayed[t] = q[t] * q_scale * exp(c_t)
+ * (fp32 [T, channels], channels = heads * dim) and totals[piece] = exp(c_last) for the pieces
+ * piece_start_loc[i] .. piece_start_loc[i + 1] - 1; the caller adds q_decayed S_start to the
+ * outputs of each piece (a matrix product).  vla_seq_gla_combine_states walks one sequence's
+ * pieces: state[slots[i]] <- totals[pieces[i]] (per key channel) * state[slots[i - 1]] +
+ * state[slots[i]] for i = 1 .. count - 1, then state[final_slot] <- state[slots[count - 1]]. */
+int vla_seq_gla_piece_prefix(float* q_decayed, float* totals, const void* q, int64_t q_stride,
+                             const float* log_decay, const int* piece_start_loc, float q_scale,
+                             int num_pieces, int channels, int dtype, void* stream);
+int vla_seq_gla_combine_states(float* state, const int* slots, const int* pieces,
+                               const float* totals, int count, int final_slot, int num_slots,
+                               int heads, int dim, int vdim, void* stream);
+
 /* The same attention for 16-bit activations, tiled over runs of 32 query rows of a sequence on
  * the matrix cores: rows query_start_loc[b] .. query_start_loc[b + 1] - 1 of sequence b sit at
  * positions context_lens[b] ...  dim must be a multiple of 32, at most 128

@@ -183,6 +183,22 @@ def test_long_decoding_over_many_windows_and_pages(tmp_path):
     s.check(torch.cat(got), toks)
 
 
+def test_long_prompts_walk_the_recurrence_in_pieces(tmp_path, monkeypatch):
+    """Prompts long enough for the recurrent layer to cut them into pieces (cut short here so the
+    reference stays quick), whole and in large portions beside a decoding request, against the
+    reference; then decoding goes on from the state the pieces left."""
+    from vllm_legacy_amd.attention.recurrent import GatedLinearRecurrence
+    monkeypatch.setattr(GatedLinearRecurrence, "PIECE_ROWS", 16)
+    s = Served(tmp_path, "loop3", torch.float32, num_blocks=80)
+    a, b = tokens_of(s.cfg, 75, 5), tokens_of(s.cfg, 110, 6)
+    got_a = [s.step([("a", a[:70])])["a"]] + [s.step([("a", a[t:t + 1])])["a"] for t in range(70, 75)]
+    s.check(torch.cat(got_a), a, "whole + decode")
+    s.end("a")
+    got_b = [s.step([("b", b[:45])])["b"], s.step([("b", b[45:104]), ("a", a[:3])])["b"]]
+    got_b += [s.step([("b", b[t:t + 1])])["b"] for t in range(104, 110)]
+    s.check(torch.cat(got_b), b, "portions + decode")
+
+
 def test_a_batch_does_not_change_a_request(tmp_path):
     """The same request alone and beside two others: equal beyond rounding (float32)."""
     s = Served(tmp_path, "odd", torch.float32)

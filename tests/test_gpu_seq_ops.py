@@ -488,3 +488,47 @@ def test_gla_carries_a_far_token(decode, scan_kernel):
     else:
         last = run_scan(q, k, v, ln_a, state, [0, n], [0], [0], H, D, V, 1.0)[n - 1, 0]
     close(last, 2.0 * v[3], 1e-5)
+
+
+@pytest.mark.parametrize("piece_rows", [8, 32])
+def test_recurrent_layer_cuts_long_runs_into_pieces(piece_rows, monkeypatch):
+    """The layer as the model calls it: runs of at least two pieces are walked piece-parallel
+    (zero-state walks, a matrix product for the missing start state, a chain over the pieces'
+    states), next to a short run and a single row, with one cut sequence continuing a context.
+    Everything must equal the one long walk."""
+    from vllm_legacy_amd.attention.batch import SequenceBatch
+    from vllm_legacy_amd.attention.recurrent import GatedLinearRecurrence
+    monkeypatch.setattr(GatedLinearRecurrence, "PIECE_ROWS", piece_rows)
+    H, D, V, rank, tau, eps = 2, 12, 20, 3, 5.0, 1e-5
+    layer = GatedLinearRecurrence(H, D, V, tau, eps)
+    g = torch.Generator().manual_seed(piece_rows)
+    lens, ctx = [5 * piece_rows + 3, 3, 2 * piece_rows, 1], [0, 4, 7, 9]
+    slots = [2, 0, 3, 1]
+    state = torch.randn(GatedLinearRecurrence.get_state_shape(4, H, D, V), generator=g).to(DEV)
+    w2, bias = torch.randn(H * D, rank, generator=g) * 0.5, torch.randn(H * D, generator=g) + 2
+    norm_w = torch.randn(V, generator=g)
+
+    def mk(n):
+        return [torch.randn(n, w, generator=g) for w in (H * D, H * D, H * V, H * V, rank)]     # q k v gate y
+    seqs = [mk(c + n) for c, n in zip(ctx, lens)]
+
+    def run(batch_lens, batch_ctx, batch_slots, parts):
+        b = SequenceBatch.build(batch_lens, batch_ctx, [[0] * 64] * len(batch_lens), batch_slots, 16, DEV)
+        q, k, v, gate, y = (torch.cat([p[i] for p in parts]).to(DEV) for i in range(5))
+        out = torch.empty(q.shape[0], H * V, device=DEV)
+        layer(out, q, k, v, gate, y, w2.to(DEV), bias.to(DEV), norm_w.to(DEV), state, b, 0.8)
+        return out.cpu()
+
+    for b_, c in enumerate(ctx):              # contexts, one sequence at a time
+        if c:
+            run([c], [0], [slots[b_]], [[t[:c] for t in seqs[b_]]])
+    got = run(lens, ctx, slots, [[t[c:] for t in s] for s, c in zip(seqs, ctx)])
+    at = 0
+    for b_, (c, n) in enumerate(zip(ctx, lens)):
+        q, k, v, gate, y = (t.to(R.F) for t in seqs[b_])
+        ln_a = R.log_decay(y, w2.to(R.F), bias.to(R.F), tau)
+        o, st = R.gated_linear_attention(q * D**-0.5, k, v, ln_a, H, D, V)
+        want = R.gated_head_norm(o, norm_w.to(R.F), gate, eps, 0.8)[c:]
+        close(got[at:at + n], want, 3e-5)
+        close(state[slots[b_]], st, 3e-5)
+        at += n

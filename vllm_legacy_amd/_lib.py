@@ -54,6 +54,7 @@ SEQ_EXPORTS = [
     "vla_seq_key_cache_write", "vla_seq_window_attention", "vla_seq_gla_log_decay",
     "vla_seq_gla_scan", "vla_seq_set_window_kernel", "vla_seq_window_attention_tiles",
     "vla_seq_window_attention_tiles_supported", "vla_seq_set_scan_kernel",
+    "vla_seq_gla_piece_prefix", "vla_seq_gla_combine_states",
 ]
 _seq_lib = None
 
@@ -88,6 +89,8 @@ def seq_lib():
                                                i, i, i, i, f, f, f, f, i, p]
         L.vla_seq_set_window_kernel.argtypes = [i]
         L.vla_seq_set_scan_kernel.argtypes = [i]
+        L.vla_seq_gla_piece_prefix.argtypes = [p, p, p, i64, p, p, f, i, i, i, p]
+        L.vla_seq_gla_combine_states.argtypes = [p, p, p, p, i, i, i, i, i, i, p]
         L.vla_seq_window_attention_tiles_supported.argtypes = [i, i]
         L.vla_seq_window_attention_tiles.argtypes = [p, i64, p, i64, p, i64, p, p, i, p, p, p, i, i, i,
                                                      i, i, i, i, i, f, f, f, f, i, p]

@@ -223,3 +223,35 @@ def gla_scan(o: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
             _rows(v, H * V), log_decay.data_ptr(), state.data_ptr(), query_start_loc.data_ptr(),
             context_lens.data_ptr(), state_slots.data_ptr(), float(q_scale), B, slots, int(max_query_len), H, D, V,
             _dt(q.dtype), _stream(q.device)), "gla_scan")
+
+
+def gla_piece_prefix(q_decayed: torch.Tensor, totals: torch.Tensor, q: torch.Tensor, log_decay: torch.Tensor,
+                     piece_start_loc: torch.Tensor, q_scale: float) -> None:
+    """q_decayed fp32 [T, C] = q * q_scale * exp(running sum of log_decay within each piece);
+    totals fp32 [pieces, C] = exp(the piece's whole sum)."""
+    _gpu(q_decayed, totals, q, log_decay, piece_start_loc)
+    T, Cn = log_decay.shape
+    P = piece_start_loc.numel() - 1
+    assert q_decayed.dtype == torch.float32 and q_decayed.is_contiguous() and q_decayed.shape == (T, Cn)
+    assert totals.dtype == torch.float32 and totals.is_contiguous() and totals.shape == (P, Cn)
+    assert log_decay.dtype == torch.float32 and log_decay.is_contiguous()
+    assert piece_start_loc.dtype == torch.int32 and piece_start_loc.is_contiguous()
+    with torch.cuda.device(q.device):
+        seq_check(_lib.seq_lib().vla_seq_gla_piece_prefix(
+            q_decayed.data_ptr(), totals.data_ptr(), q.data_ptr(), _rows(q, Cn), log_decay.data_ptr(),
+            piece_start_loc.data_ptr(), float(q_scale), P, Cn, _dt(q.dtype), _stream(q.device)), "gla_piece_prefix")
+
+
+def gla_combine_states(state: torch.Tensor, slots: torch.Tensor, pieces: torch.Tensor, totals: torch.Tensor,
+                       final_slot: int) -> None:
+    _gpu(state, slots, pieces, totals)
+    n, H, D, V = state.shape
+    assert state.dtype == torch.float32 and state.is_contiguous() and totals.dtype == torch.float32
+    assert totals.is_contiguous() and totals.shape[1] == H * D
+    for t in (slots, pieces):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    assert slots.numel() == pieces.numel()
+    with torch.cuda.device(state.device):
+        seq_check(_lib.seq_lib().vla_seq_gla_combine_states(
+            state.data_ptr(), slots.data_ptr(), pieces.data_ptr(), totals.data_ptr(), slots.numel(),
+            int(final_slot), n, H, D, V, _stream(state.device)), "gla_combine_states")

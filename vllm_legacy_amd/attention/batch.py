@@ -8,7 +8,7 @@ Gfx950PagedAttentionMetadata (prompts first, decode tokens after them) describes
 the paged-attention decode kernels take; `SequenceBatch.build` is what an engine calls per step.
 """
 from dataclasses import dataclass
-from typing import List, Sequence
+from typing import List, Optional, Sequence
 
 import torch
 
@@ -26,6 +26,10 @@ class SequenceBatch:
     state_slots: torch.Tensor       # int32 [B] recurrent-state slot of each sequence
     max_query_len: int
     max_seq_len: int                # longest context + query of the step
+    # host copies of the per-sequence numbers, for layers that plan their launches on the host
+    host_query_lens: Optional[List[int]] = None
+    host_context_lens: Optional[List[int]] = None
+    host_state_slots: Optional[List[int]] = None
 
     @staticmethod
     def build(query_lens: Sequence[int], context_lens: Sequence[int],
@@ -66,4 +70,6 @@ class SequenceBatch:
             query_start_loc=dev(starts, torch.int32), context_lens=dev(list(context_lens), torch.int32),
             block_tables=tables.to(device, non_blocking=True),
             state_slots=dev(list(state_slots), torch.int32), max_query_len=max(query_lens),
-            max_seq_len=max(int(c) + int(n) for c, n in zip(context_lens, query_lens)))
+            max_seq_len=max(int(c) + int(n) for c, n in zip(context_lens, query_lens)),
+            host_query_lens=[int(n) for n in query_lens], host_context_lens=[int(c) for c in context_lens],
+            host_state_slots=[int(x) for x in state_slots])

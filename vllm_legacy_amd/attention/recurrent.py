@@ -5,8 +5,15 @@ a_t = sigmoid(z_t)^(1 / tau) from a low-rank projection z_t = W2 y_t + b.  The s
 fp32 tensor [num_slots, heads, dim, vdim] that the engine's cache manager hands out by slot; a
 sequence whose context length is 0 starts from zero whatever its slot held before.  The output of
 each head is RMS-normed over vdim, gated with silu and scaled before the output projection.
+
+A long run of rows (a prompt, a large portion) is cut into pieces of PIECE_ROWS rows that are
+walked at the same time, each from a zero state in a scratch slot behind the sequences' slots;
+the state a piece should have started from then reaches its outputs through one batched matrix
+product (o_t += (q_t exp(c_t))^T S_start, c_t the log decays summed from the piece's first row)
+and the pieces' states are chained by a cheap walk.  The result is the long walk's, to rounding.
 Kernels: csrc/seq_linear_recurrence.hip, csrc/seq_stream_kernels.hip.
 """
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -17,6 +24,9 @@ from vllm_legacy_amd.attention.batch import SequenceBatch
 
 
 class GatedLinearRecurrence(nn.Module):
+    # rows of a piece; runs of at least two pieces are cut (VLA_GLA_PIECE_ROWS: another size, for studies)
+    PIECE_ROWS = int(os.environ.get("VLA_GLA_PIECE_ROWS", "256"))
+    SCRATCH_SLOTS = 64      # state slots behind the sequences' own, for the pieces of a step
 
     def __init__(self, num_heads: int, head_dim: int, value_dim: int, tau: float, eps: float,
                  q_scale: Optional[float] = None) -> None:
@@ -28,7 +38,36 @@ class GatedLinearRecurrence(nn.Module):
     @staticmethod
     def get_state_shape(num_slots: int, num_heads: int, head_dim: int,
                         value_dim: int) -> Tuple[int, ...]:
-        return (num_slots, num_heads, head_dim, value_dim)
+        """num_slots sequence slots, then SCRATCH_SLOTS slots that only live within a step."""
+        return (num_slots + GatedLinearRecurrence.SCRATCH_SLOTS, num_heads, head_dim, value_dim)
+
+    def _plan_pieces(self, batch: SequenceBatch, num_slots: int):
+        """None when no run of the step is long enough (or scratch would not suffice); else
+        (piece_start_loc, piece_context, piece_slots, [per cut sequence: (first piece, count, own
+        slot, first row)])."""
+        q, c, sl = batch.host_query_lens, batch.host_context_lens, batch.host_state_slots
+        L = self.PIECE_ROWS
+        if q is None or max(q) < 2 * L:
+            return None
+        first_scratch = num_slots - self.SCRATCH_SLOTS
+        starts, ctx, slots, cut, row, scratch = [0], [], [], [], 0, first_scratch
+        for n, cb, sb in zip(q, c, sl):
+            if n < 2 * L:
+                ctx.append(cb)
+                slots.append(sb)
+                starts.append(starts[-1] + n)
+            else:
+                count = (n + L - 1) // L
+                if scratch + count > num_slots:
+                    return None
+                cut.append((len(ctx), count, sb, row, cb))
+                for i in range(count):
+                    ctx.append(cb if i == 0 else 0)
+                    slots.append(scratch + i)
+                    starts.append(starts[-1] + min(L, n - i * L))
+                scratch += count
+            row += n
+        return starts, ctx, slots, cut
 
     def forward(self, out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                 gate: torch.Tensor, y: torch.Tensor, w2: torch.Tensor, bias: Optional[torch.Tensor],
@@ -40,7 +79,44 @@ class GatedLinearRecurrence(nn.Module):
         log_decay = torch.empty((T, H * D), dtype=torch.float32, device=q.device)
         ops.gla_log_decay(log_decay, y, w2, bias, self.inv_tau)
         o = torch.empty((T, H, V), dtype=torch.float32, device=q.device)
-        ops.gla_scan(o, q, k, v, log_decay, state, batch.query_start_loc, batch.context_lens,
-                     batch.state_slots, self.q_scale, batch.max_query_len)
+        plan = self._plan_pieces(batch, state.shape[0])
+        if plan is None:
+            ops.gla_scan(o, q, k, v, log_decay, state, batch.query_start_loc, batch.context_lens,
+                         batch.state_slots, self.q_scale, batch.max_query_len)
+        else:
+            self._scan_in_pieces(o, q, k, v, log_decay, state, plan)
         ops.gated_head_rms_norm(out, o, norm_weight, gate, self.eps, out_scale)
         return out
+
+    def _scan_in_pieces(self, o, q, k, v, log_decay, state, plan) -> None:
+        starts, ctx, slots, cut = plan
+        dev, L = q.device, self.PIECE_ROWS
+        H, D, V = self.num_heads, self.head_dim, self.value_dim
+
+        def i32(x):
+            return torch.as_tensor(x, dtype=torch.int32).to(dev, non_blocking=True)
+
+        for first, count, own, row, cb in cut:      # a continuing sequence starts from its state
+            if cb > 0:
+                state[slots[first]].copy_(state[own])
+        start_loc = i32(starts)
+        ops.gla_scan(o, q, k, v, log_decay, state, start_loc, i32(ctx), i32(slots), self.q_scale,
+                     max(b - a for a, b in zip(starts, starts[1:])))
+        q_decayed = torch.empty((q.shape[0], H * D), dtype=torch.float32, device=dev)
+        totals = torch.empty((len(ctx), H * D), dtype=torch.float32, device=dev)
+        ops.gla_piece_prefix(q_decayed, totals, q, log_decay, start_loc, self.q_scale)
+        for first, count, own, row, cb in cut:
+            piece_slots = slots[first:first + count]
+            ops.gla_combine_states(state, i32(piece_slots), i32(list(range(first, first + count))), totals, own)
+            n = starts[first + count] - starts[first]
+            full = n // L                           # pieces of exactly L rows
+            # pieces 1 .. full - 1 start from the states at the end of pieces 0 .. full - 2
+            if full > 1:
+                r0, r1 = row + L, row + full * L
+                s_start = state[piece_slots[0]:piece_slots[0] + full - 1]              # [p, H, D, V]
+                qd = q_decayed[r0:r1].view(full - 1, L, H, D).permute(0, 2, 1, 3)       # [p, H, L, D]
+                o[r0:r1].view(full - 1, L, H, V).permute(0, 2, 1, 3).add_(torch.matmul(qd, s_start))
+            if n > full * L:                        # the shorter last piece
+                r0 = row + full * L
+                qd = q_decayed[r0:row + n].view(n - full * L, H, D).permute(1, 0, 2)    # [H, l, D]
+                o[r0:row + n].permute(1, 0, 2).add_(torch.matmul(qd, state[piece_slots[full - 1]]))

@@ -306,6 +306,53 @@ __global__ __launch_bounds__(256) void gla_scan_block_kernel(
   }
 }
 
+
+// ---- pieces of a long run of rows, walked in parallel ------------------------------------------
+// A run of many rows of one sequence is cut into pieces.  Every piece is walked from a zero state
+// (the first from the sequence's own), all at once; that leaves, per piece, outputs that lack the
+// state the piece should have started from, and the state the piece adds.  With
+// c_t = sum of the log decays from the piece's first row to row t,
+//   o_t += (q_t * exp(c_t))^T S_start          (a matrix product per piece and head)
+//   S_end = diag(exp(c_last)) S_start + S_piece (a cheap walk over the pieces)
+// give exactly what the one long walk computes.  Every exponent is <= 0: nothing can overflow.
+//
+// gla_piece_prefix_kernel: c_t by a running sum over the piece's rows, one thread per (piece,
+// channel); writes q_t * q_scale * exp(c_t) and, per piece, exp(c_last).
+template <class S>
+__global__ __launch_bounds__(256) void gla_piece_prefix_kernel(
+    float* __restrict__ q_decayed, float* __restrict__ totals, const typename S::T* __restrict__ q,
+    int64_t q_stride, const float* __restrict__ log_decay, const int* __restrict__ piece_start_loc,
+    float q_scale, int channels) {
+  const int piece = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= channels) return;
+  const int t0 = piece_start_loc[piece], t1 = piece_start_loc[piece + 1];
+  float sum = 0.f;
+#pragma unroll 8
+  for (int t = t0; t < t1; ++t) {
+    sum += log_decay[(int64_t)t * channels + c];
+    q_decayed[(int64_t)t * channels + c] = S::to_f32(q[(int64_t)t * q_stride + c]) * q_scale * expf(sum);
+  }
+  totals[(int64_t)piece * channels + c] = expf(sum);
+}
+
+// gla_combine_states_kernel: the pieces' states of one sequence in order; state[slots[i]] becomes
+// the state at the end of piece i, and the last one is copied to the sequence's own slot.
+__global__ __launch_bounds__(256) void gla_combine_states_kernel(
+    float* __restrict__ state, const int* __restrict__ slots, const int* __restrict__ pieces,
+    const float* __restrict__ totals, int count, int final_slot, int heads, int dim, int vdim) {
+  const int64_t per = (int64_t)heads * dim * vdim;
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= per) return;
+  const int channel = (int)(e / vdim);            // h * dim + d
+  float run = state[slots[0] * per + e];
+  for (int i = 1; i < count; ++i) {
+    run = totals[(int64_t)pieces[i] * heads * dim + channel] * run + state[slots[i] * per + e];
+    state[slots[i] * per + e] = run;
+  }
+  state[final_slot * per + e] = run;
+}
+
 }  // namespace
 }  // namespace seq
 }  // namespace vla
@@ -349,8 +396,15 @@ extern "C" int vla_seq_gla_scan(float* o, const void* q, int64_t q_stride, const
     // writing the state, which wide slices do in fewer, fuller workgroups.  Measured on
     // 16 heads x 64 x 128: 4096 tokens 1.45 ms at 16 columns against 2.03 ms at 64; 64 sequences
     // of one token 40 us at 64 columns against 120 us at 16.
+    // Every slice of a head fetches the head's q, k and decays again, so slices are only as narrow
+    // as it takes to give every CU a workgroup.
     int cols = g_scan_cols.load(std::memory_order_relaxed);
-    if (cols == 0) cols = (max_query_len > 0 && max_query_len <= 4) ? 64 : 16;
+    if (cols == 0) {
+      cols = 16;
+      if (max_query_len > 0 && max_query_len <= 4) cols = 64;
+      else if ((int64_t)num_seqs * heads * ((vdim + 63) / 64) >= 256) cols = 64;
+      else if ((int64_t)num_seqs * heads * ((vdim + 31) / 32) >= 256) cols = 32;
+    }
     const int vb = vdim < cols ? vdim : cols;
     const int slices = (vdim + vb - 1) / vb;
     int groups = 256 / vb;
@@ -450,5 +504,36 @@ extern "C" int vla_seq_gla_scan(float* o, const void* q, int64_t q_stride, const
 extern "C" int vla_seq_set_scan_kernel(int mode) {
   if (mode < 0 || mode > 1) return VLA_ERR_ARG;
   g_scan_kernel.store(mode, std::memory_order_relaxed);
+  return VLA_OK;
+}
+
+extern "C" int vla_seq_gla_piece_prefix(float* q_decayed, float* totals, const void* q,
+                                        int64_t q_stride, const float* log_decay,
+                                        const int* piece_start_loc, float q_scale, int num_pieces,
+                                        int channels, int dtype, void* stream) {
+  if (num_pieces == 0) return VLA_OK;
+  if (!q_decayed || !totals || !q || !log_decay || !piece_start_loc || num_pieces < 0 ||
+      channels <= 0 || q_stride < channels)
+    return VLA_ERR_ARG;
+  return with_dtype(dtype, [&](auto s) {
+    using S = decltype(s);
+    gla_piece_prefix_kernel<S><<<dim3((channels + 255) / 256, num_pieces), 256, 0, (hipStream_t)stream>>>(
+        q_decayed, totals, (const typename S::T*)q, q_stride, log_decay, piece_start_loc, q_scale, channels);
+    VLA_SEQ_HIP_CHECK(hipGetLastError());
+    return VLA_OK;
+  });
+}
+
+extern "C" int vla_seq_gla_combine_states(float* state, const int* slots, const int* pieces,
+                                          const float* totals, int count, int final_slot,
+                                          int num_slots, int heads, int dim, int vdim, void* stream) {
+  if (count == 0) return VLA_OK;
+  if (!state || !slots || !pieces || !totals || count < 0 || final_slot < 0 || final_slot >= num_slots ||
+      heads <= 0 || dim <= 0 || vdim <= 0)
+    return VLA_ERR_ARG;
+  const int64_t per = (int64_t)heads * dim * vdim;
+  gla_combine_states_kernel<<<(unsigned)((per + 255) / 256), 256, 0, (hipStream_t)stream>>>(
+      state, slots, pieces, totals, count, final_slot, heads, dim, vdim);
+  VLA_SEQ_HIP_CHECK(hipGetLastError());
   return VLA_OK;
 }

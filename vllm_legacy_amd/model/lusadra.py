@@ -256,6 +256,7 @@ class LusadraForCausalLM(nn.Module):
         for spec in self.cache_spec():
             keys = torch.zeros(WindowedKeyAttention.get_cache_shape(num_blocks, block_size, *spec["keys"]),
                                dtype=self.dtype, device=dev)
+            # (the recurrent layer adds its scratch slots behind the sequences' own)
             state = torch.zeros(GatedLinearRecurrence.get_state_shape(num_slots, *spec["state"]),
                                 dtype=torch.float32, device=dev)
             caches.append((keys, state))
