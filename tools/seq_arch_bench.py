@@ -145,6 +145,13 @@ def run(args):
                    nbytes=T * (2.0 * (2 * Hr * Dr + Hr * Vr) + 4.0 * Hr * Dr + 4.0 * Hr * Vr) + 8.0 * nseq * Hr * Dr * Vr,
                    note="a recurrence: the walk over a sequence's tokens is serial")
             y = torch.randn(T, lay.rank, device=dev, dtype=dt)
+            og2 = torch.empty(T, Hr * Vr, device=dev, dtype=dt)
+            # the layer as the model calls it: log decays, the walk (long runs in pieces), norm + gate
+            sec = timed(lambda: lay.recur(og2, qr, kr, vr, vr, y, lay.w_a2.data, lay.b_a2.data, lay.recur_norm.data,
+                                          state, batch, 0.5), 5 if tag == "prefill" else 20)
+            record(kern, f"lusadra.recurrent_layer.{tag}", sec, peak=FMA_F32, flops=4.0 * T * Hr * Dr * Vr,
+                   nbytes=T * (2.0 * (2 * Hr * Dr + 3 * Hr * Vr) + 2.0 * lay.rank) + 8.0 * nseq * Hr * Dr * Vr,
+                   note="log decays + walk + gated norm; runs of 512 rows and more are walked in pieces of 256")
             sec = timed(lambda: sops.gla_log_decay(ld, y, lay.w_a2.data, lay.b_a2.data, 1 / 16.0))
             record(kern, f"lusadra.gla_log_decay.{tag}", sec, nbytes=4.0 * T * Hr * Dr + 2.0 * T * lay.rank)
             og = torch.empty(T, Hr * Vr, device=dev, dtype=dt)
