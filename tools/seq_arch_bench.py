@@ -39,9 +39,9 @@ SIZES = {
 def lusadra_config(s, layers, vocab):
     layer = {"type": "parallel",
              "mixer": {"left": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"],
-                                "mask": {"size": s["window"]}, "q_temp": {"coef": 0.3, "every": 512},
+                                "mask": {"size": s["window"]}, "q_temp": {"coef": 0.25, "every": 512},
                                 "scale": s["dim"]**-0.5},
-                       "right": {"heads": s["r_heads"], "dim": s["r_dim"], "vdim": s["r_vdim"], "tau": 16.0},
+                       "right": {"heads": s["r_heads"], "dim": s["r_dim"], "vdim": s["r_vdim"], "tau": 8.0},
                        "left_scale": 0.5, "right_scale": 0.5},
              "mlp": {"kind": "dense", "ff": s["ff"]}}
     return {"architecture": "Lusadra", "vocab": vocab, "width": s["width"], "norm": {"eps": 1e-5},
@@ -119,10 +119,10 @@ def run(args):
                 sec = timed(lambda: sops.window_attention_tiles(out, q, gate, keys, batch.block_tables,
                                                                 batch.query_start_loc, batch.context_lens,
                                                                 batch.max_query_len, lay.attn.slopes, H, W, D**-0.5,
-                                                                0.3, 512.0, 0.5), 5)
+                                                                0.25, 512.0, 0.5), 5)
             else:
                 sec = timed(lambda: sops.window_attention(out, q, gate, keys, batch.block_tables, batch.token_seq,
-                                                          batch.positions, lay.attn.slopes, H, W, D**-0.5, 0.3, 512.0,
+                                                          batch.positions, lay.attn.slopes, H, W, D**-0.5, 0.25, 512.0,
                                                           0.5), 20)
             if tag == "prefill":
                 pairs = sum(min(W, p + 1) for p in range(T))
@@ -152,7 +152,7 @@ def run(args):
             record(kern, f"lusadra.recurrent_layer.{tag}", sec, peak=FMA_F32, flops=4.0 * T * Hr * Dr * Vr,
                    nbytes=T * (2.0 * (2 * Hr * Dr + 3 * Hr * Vr) + 2.0 * lay.rank) + 8.0 * nseq * Hr * Dr * Vr,
                    note="log decays + walk + gated norm; runs of 512 rows and more are walked in pieces of 256")
-            sec = timed(lambda: sops.gla_log_decay(ld, y, lay.w_a2.data, lay.b_a2.data, 1 / 16.0))
+            sec = timed(lambda: sops.gla_log_decay(ld, y, lay.w_a2.data, lay.b_a2.data, 1 / 8.0))
             record(kern, f"lusadra.gla_log_decay.{tag}", sec, nbytes=4.0 * T * Hr * Dr + 2.0 * T * lay.rank)
             og = torch.empty(T, Hr * Vr, device=dev, dtype=dt)
             sec = timed(lambda: sops.gated_head_rms_norm(og, o, lay.recur_norm.data, vr, 1e-5, 0.5))
