@@ -51,7 +51,7 @@ def test_config_reader_refuses_what_it_does_not_know():
 
 
 def test_registry():
-    assert "Lusadra" in registry.supported_architectures()
+    assert {"Lusadra", "LlamaDecodeStack"} <= set(registry.supported_architectures())
     model_cls, config_cls = registry.resolve("Lusadra")
     assert model_cls.__name__ == "LusadraForCausalLM" and config_cls is LusadraConfig
     with pytest.raises(ValueError):

@@ -11,6 +11,8 @@
   trace replay (given steps instead of scheduled ones, logits to files)
                                               engine/trace_replay.py, bin/trace_run
   command line                                engine/cli.py
+  the Llama decode stack behind the same protocol
+                                              engine/llama_adapter.py
 """
 from .cache_manager import CacheManager  # noqa: F401
 from .llm_engine import EngineConfig, LLMEngine, RequestOutput  # noqa: F401

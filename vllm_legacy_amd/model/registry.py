@@ -11,6 +11,8 @@ import torch
 # architecture -> (module, model class, config class)
 _MODELS: Dict[str, Tuple[str, str, str]] = {
     "Lusadra": ("vllm_legacy_amd.model.lusadra", "LusadraForCausalLM", "LusadraConfig"),
+    # the synthetic-weight Llama stack behind the engine's model protocol
+    "LlamaDecodeStack": ("vllm_legacy_amd.engine.llama_adapter", "PagedLlamaForEngine", "LlamaEngineConfig"),
 }
 
 
@@ -41,13 +43,15 @@ def architecture_of(config: Dict) -> str:
 
 
 def load_model(model_dir: str, dtype: torch.dtype = torch.bfloat16, device="cuda"):
-    """Build the model a folder's config.json names and fill it from its model.safetensors."""
+    """Build the model a folder's config.json names and fill it from its model.safetensors
+    (a folder without one gets the model's own random weights: synthetic stacks)."""
     from vllm_legacy_amd.model_loader.safetensors_file import load_safetensors
     with open(os.path.join(model_dir, "config.json")) as f:
         raw = json.load(f)
     model_cls, config_cls = resolve(architecture_of(raw))
     cfg = config_cls.from_dict(raw)
     model = model_cls(cfg, dtype=dtype, device=device)
-    tensors = load_safetensors(os.path.join(model_dir, "model.safetensors"))
-    model.load_weights(tensors)
+    weights = os.path.join(model_dir, "model.safetensors")
+    if os.path.exists(weights):
+        model.load_weights(load_safetensors(weights))
     return model
