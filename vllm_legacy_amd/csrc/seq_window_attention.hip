@@ -531,17 +531,16 @@ __global__ __launch_bounds__(64 * kRowWaves) void window_attention_heads_kernel(
     const typename S::T* __restrict__ cache, const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ token_seq, const int64_t* __restrict__ positions,
     const float* __restrict__ slopes, int heads, int kv_heads, int block_size, int num_blocks,
-    int window, float scale, float temp_coef, float temp_every, float out_scale) {
+    int window, float scale, float temp_coef, float temp_every, float out_scale, int merge_heads) {
   using T = typename S::T;
   using M = Mfma8<S>;
   constexpr int D = 32 * DB;
-  constexpr int KROW = D + 4, TROW = kTile + 4;
-  constexpr int WAVE_ELEMS = kTile * KROW + D * TROW;     // one wave's two tiles, in elements
+  constexpr int KROW = D + 4;
+  constexpr int WAVE_ELEMS = kTile * KROW;                // one wave's tile, in elements
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int hf = lane >> 5, c = lane & 31;
   T* k_lds = reinterpret_cast<T*>(smem) + (size_t)w * WAVE_ELEMS;
-  T* kt_lds = k_lds + kTile * KROW;
   const int t = blockIdx.x;
   const int group = heads / kv_heads;
   const int chunks = (group + 31) / 32;
@@ -602,11 +601,6 @@ __global__ __launch_bounds__(64 * kRowWaves) void window_attention_heads_kernel(
       const int i = lane + kWave * u;
       const int r = i / (D / 4), v = i % (D / 4);
       *reinterpret_cast<u32x2*>(k_lds + r * KROW + 4 * v) = x[u];
-      uint16_t* col = reinterpret_cast<uint16_t*>(kt_lds) + (4 * v) * TROW + r;
-      col[0] = (uint16_t)(x[u][0] & 0xffffu);
-      col[TROW] = (uint16_t)(x[u][0] >> 16);
-      col[2 * TROW] = (uint16_t)(x[u][1] & 0xffffu);
-      col[3 * TROW] = (uint16_t)(x[u][1] >> 16);
     }
     if (j0 + kRowWaves * kTile <= p) fetch(j0 + kRowWaves * kTile);
     wave_sync();
@@ -653,7 +647,12 @@ __global__ __launch_bounds__(64 * kRowWaves) void window_attention_heads_kernel(
       const u32x2 lo2 = {lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16)};
 #pragma unroll
       for (int n = 0; n < DB; ++n) {
-        const u32x2 a = *reinterpret_cast<const u32x2*>(kt_lds + (32 * n + c) * TROW + 8 * s8 + 4 * hf);
+        // K^T operand from the row-major tile: dim 32 n + c of keys 8 s8 + 4 hf .. + 3 (a
+        // transposed copy of the tile costs 16-bit scatter writes that collide in the LDS banks
+        // and, with eight waves a CU, took most of the kernel's time)
+        const uint16_t* col = reinterpret_cast<const uint16_t*>(k_lds) + (8 * s8 + 4 * hf) * KROW + 32 * n + c;
+        const u32x2 a = {(uint32_t)col[0] | ((uint32_t)col[KROW] << 16),
+                         (uint32_t)col[2 * KROW] | ((uint32_t)col[3 * KROW] << 16)};
         o[n] = M::run(a, hi, o[n]);
         o[n] = M::run(a, lo2, o[n]);
       }
@@ -665,7 +664,7 @@ __global__ __launch_bounds__(64 * kRowWaves) void window_attention_heads_kernel(
   __syncthreads();
   float* merge = reinterpret_cast<float*>(smem);
   if (live) {
-    float* mine = merge + ((size_t)w * 32 + c) * (2 + D);
+    float* mine = merge + ((size_t)w * merge_heads + c) * (2 + D);
     if (hf == 0) {
       mine[0] = m;
       mine[1] = l;
@@ -679,10 +678,10 @@ __global__ __launch_bounds__(64 * kRowWaves) void window_attention_heads_kernel(
   for (int i = tid; i < nh * D; i += 64 * kRowWaves) {
     const int hh = i / D, d = i - hh * D;
     float mm = -INFINITY;
-    for (int ww = 0; ww < kRowWaves; ++ww) mm = fmaxf(mm, merge[((size_t)ww * 32 + hh) * (2 + D)]);
+    for (int ww = 0; ww < kRowWaves; ++ww) mm = fmaxf(mm, merge[((size_t)ww * merge_heads + hh) * (2 + D)]);
     float ll = 0.f, ov = 0.f;
     for (int ww = 0; ww < kRowWaves; ++ww) {
-      const float* src = merge + ((size_t)ww * 32 + hh) * (2 + D);
+      const float* src = merge + ((size_t)ww * merge_heads + hh) * (2 + D);
       const float f = src[0] == -INFINITY ? 0.f : expf(src[0] - mm);
       ll += src[1] * f;
       ov += src[2 + d] * f;
@@ -697,10 +696,10 @@ __global__ __launch_bounds__(64 * kRowWaves) void window_attention_heads_kernel(
 }
 
 template <class S, int DB>
-size_t heads_kernel_lds() {
+size_t heads_kernel_lds(int merge_heads) {
   constexpr int D = 32 * DB;
-  const size_t tiles = (size_t)kRowWaves * (kTile * (D + 4) + D * (kTile + 4)) * sizeof(typename S::T);
-  const size_t merge = (size_t)kRowWaves * 32 * (2 + D) * sizeof(float);
+  const size_t tiles = (size_t)kRowWaves * kTile * (D + 4) * sizeof(typename S::T);
+  const size_t merge = (size_t)kRowWaves * merge_heads * (2 + D) * sizeof(float);
   return tiles > merge ? tiles : merge;
 }
 
@@ -711,7 +710,9 @@ int launch_heads_one(dim3 grid, hipStream_t stream, typename S::T* out, int64_t 
                      int max_blocks, const int* token_seq, const int64_t* positions,
                      const float* slopes, int heads, int kv_heads, int block_size, int num_blocks,
                      int window, float scale, float temp_coef, float temp_every, float out_scale) {
-  const size_t lds = heads_kernel_lds<S, DB>();
+  const int group = heads / kv_heads;
+  const int merge_heads = group < 32 ? group : 32;
+  const size_t lds = heads_kernel_lds<S, DB>(merge_heads);
   static std::atomic<size_t> allowed{64 * 1024};   // raised once per kernel, not per launch
   if (lds > allowed.load(std::memory_order_relaxed)) {
     VLA_SEQ_HIP_CHECK(hipFuncSetAttribute(
@@ -722,7 +723,7 @@ int launch_heads_one(dim3 grid, hipStream_t stream, typename S::T* out, int64_t 
   window_attention_heads_kernel<S, DB><<<grid, 64 * kRowWaves, lds, stream>>>(
       out, out_stride, q, q_stride, gate, gate_stride, cache, block_tables, max_blocks, token_seq,
       positions, slopes, heads, kv_heads, block_size, num_blocks, window, scale, temp_coef,
-      temp_every, out_scale);
+      temp_every, out_scale, merge_heads);
   VLA_SEQ_HIP_CHECK(hipGetLastError());
   return VLA_OK;
 }
