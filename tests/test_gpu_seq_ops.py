@@ -532,3 +532,23 @@ def test_recurrent_layer_cuts_long_runs_into_pieces(piece_rows, monkeypatch):
         close(got[at:at + n], want, 3e-5)
         close(state[slots[b_]], st, 3e-5)
         at += n
+
+
+@pytest.mark.parametrize("features,offset", [(40, 0), (256, 4), (1100, 8), (4100, 0), (5632, 4), (300, 3), (302, 0)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_poly_norm_16bit_rows_aligned_or_not(features, offset, dtype):
+    """Rows inside a wider matrix: offsets that are multiples of four values take the four-wide
+    kernel (rows longer than the 4096 values a workgroup keeps in registers included), others
+    and lengths that are not multiples of four the element-wise one."""
+    g = torch.Generator().manual_seed(features + offset)
+    width = (features + offset + 7) // 4 * 4
+    wide = (torch.randn(3, width, generator=g) * 1.5).to(dtype).to(DEV)
+    z = wide[:, offset:offset + features]
+    coef = torch.tensor([0.6, 0.3, -0.2, 0.05])
+    dst = torch.zeros(3, width, dtype=dtype, device=DEV)
+    ops().poly_norm(dst[:, offset:offset + features], z, coef.to(DEV), 1e-5)
+    want = R.poly_norm(z.cpu().to(R.F), coef, 1e-5)
+    ulp = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
+    close(dst[:, offset:offset + features].float(), want, 1.1 * ulp)
+    assert float(dst[:, :offset].float().abs().max() if offset else 0.0) == 0.0
+    assert float(dst[:, offset + features:].float().abs().max()) == 0.0

@@ -38,6 +38,21 @@ __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// the two 16-bit values of a packed word, and back
+template <class S>
+__device__ __forceinline__ float lo16(uint32_t w) {
+  return S::to_f32(__builtin_bit_cast(typename S::T, (uint16_t)(w & 0xffffu)));
+}
+template <class S>
+__device__ __forceinline__ float hi16(uint32_t w) {
+  return S::to_f32(__builtin_bit_cast(typename S::T, (uint16_t)(w >> 16)));
+}
+template <class S>
+__device__ __forceinline__ uint32_t pack16(float lo, float hi) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, S::from_f32(lo)) |
+         ((uint32_t)__builtin_bit_cast(uint16_t, S::from_f32(hi)) << 16);
+}
+
 // sum over a workgroup of up to 1024 threads; red holds 16 floats; every thread gets the sum
 __device__ __forceinline__ float block_sum(float v, float* red) {
   v = wave_sum(v);

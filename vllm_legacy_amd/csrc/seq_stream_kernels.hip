@@ -122,6 +122,68 @@ __global__ __launch_bounds__(kThreads) void poly_norm_kernel(
     put(c, S::to_f32(zr[c]));
 }
 
+// 16-bit rows whose length is a multiple of four and whose ends are 8-byte aligned: four values
+// per access, the row (up to 4096 values) kept in registers between the two passes.
+template <class S>
+__global__ __launch_bounds__(kThreads) void poly_norm_vec_kernel(
+    typename S::T* __restrict__ out, int64_t out_stride, const typename S::T* __restrict__ z,
+    int64_t z_stride, const float* __restrict__ coef, float eps, int features) {
+  __shared__ float red[16];
+  constexpr int STEPS = 4;
+  const typename S::T* zr = z + (int64_t)blockIdx.x * z_stride;
+  typename S::T* orow = out + (int64_t)blockIdx.x * out_stride;
+  float keep[STEPS][4];
+  float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  auto take = [&](int c, float (&v)[4]) {
+    const u32x2 w = *reinterpret_cast<const u32x2*>(zr + c);
+    v[0] = lo16<S>(w.x);
+    v[1] = hi16<S>(w.x);
+    v[2] = lo16<S>(w.y);
+    v[3] = hi16<S>(w.y);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float v2 = v[e] * v[e], v3 = v2 * v[e];
+      s1 += v2;
+      s2 += v2 * v2;
+      s3 += v3 * v3;
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < STEPS; ++i) {
+    const int c = (threadIdx.x + i * kThreads) * 4;
+    if (c < features) take(c, keep[i]);
+  }
+  for (int c = (threadIdx.x + STEPS * kThreads) * 4; c < features; c += kThreads * 4) {
+    float v[4];
+    take(c, v);
+  }
+  s1 = block_sum(s1, red);
+  s2 = block_sum(s2, red);
+  s3 = block_sum(s3, red);
+  const float n = (float)features;
+  const float k1 = coef[0] / sqrtf(s1 / n + eps), k2 = coef[1] / sqrtf(s2 / n + eps),
+              k3 = coef[2] / sqrtf(s3 / n + eps), k0 = coef[3];
+  auto put = [&](int c, const float (&v)[4]) {
+    float r[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float v2 = v[e] * v[e];
+      r[e] = k1 * v[e] + k2 * v2 + k3 * (v2 * v[e]) + k0;
+    }
+    *reinterpret_cast<u32x2*>(orow + c) = u32x2{pack16<S>(r[0], r[1]), pack16<S>(r[2], r[3])};
+  };
+#pragma unroll
+  for (int i = 0; i < STEPS; ++i) {
+    const int c = (threadIdx.x + i * kThreads) * 4;
+    if (c < features) put(c, keep[i]);
+  }
+  for (int c = (threadIdx.x + STEPS * kThreads) * 4; c < features; c += kThreads * 4) {
+    const u32x2 w = *reinterpret_cast<const u32x2*>(zr + c);
+    const float v[4] = {lo16<S>(w.x), hi16<S>(w.x), lo16<S>(w.y), hi16<S>(w.y)};
+    put(c, v);
+  }
+}
+
 // one wave per (token, head)
 template <class S>
 __global__ __launch_bounds__(kWave) void gated_head_rms_norm_kernel(
@@ -202,6 +264,15 @@ extern "C" int vla_seq_poly_norm(void* out, int64_t out_stride, const void* z, i
     return VLA_ERR_ARG;
   return with_dtype(dtype, [&](auto s) {
     using S = decltype(s);
+    if constexpr (sizeof(typename S::T) == 2) {
+      if (features % 4 == 0 && ((uintptr_t)z % 8) == 0 && ((uintptr_t)out % 8) == 0 && (z_stride % 4) == 0 &&
+          (out_stride % 4) == 0) {
+        poly_norm_vec_kernel<S><<<num_tokens, kThreads, 0, (hipStream_t)stream>>>(
+            (typename S::T*)out, out_stride, (const typename S::T*)z, z_stride, coef, eps, features);
+        VLA_SEQ_HIP_CHECK(hipGetLastError());
+        return VLA_OK;
+      }
+    }
     poly_norm_kernel<S><<<num_tokens, kThreads, 0, (hipStream_t)stream>>>(
         (typename S::T*)out, out_stride, (const typename S::T*)z, z_stride, coef, eps, features);
     VLA_SEQ_HIP_CHECK(hipGetLastError());

@@ -134,14 +134,6 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void window_attention_kernel
 constexpr int kHeadChunk = 4;
 constexpr int kPairs = kMaxDim / (2 * kWave);   // passes of 128 dims in the weighted sum
 
-template <class S>
-__device__ __forceinline__ float lo16(uint32_t w) {
-  return S::to_f32(__builtin_bit_cast(typename S::T, (uint16_t)(w & 0xffffu)));
-}
-template <class S>
-__device__ __forceinline__ float hi16(uint32_t w) {
-  return S::to_f32(__builtin_bit_cast(typename S::T, (uint16_t)(w >> 16)));
-}
 
 template <class S>
 __global__ __launch_bounds__(256) void window_attention_group_kernel(
