@@ -5,8 +5,10 @@ query i against the keys j of its window 0 <= i - j < window with an optional li
 bias slope_h * (i - j) and an optional query temperature that grows with the logarithm of the
 position, and gates the concatenated heads with a sigmoid before the output projection.  Every
 parameter is a constructor argument; `None` / 0 switch a term off.  Prompts, portions of prompts
-and decode steps take the same kernel (csrc/seq_window_attention.hip) after the step's keys have
-been written to the cache.
+and decode steps are one case: the step's keys are written to the cache, then every row reads
+its window from there (csrc/seq_window_attention.hip: matrix-core kernels for 16-bit models --
+tiles of 32 rows for runs of rows, all heads of a KV group at once for single rows -- and fp32
+kernels for any dtype and head size).
 """
 import os
 from typing import List, Optional, Tuple

@@ -13,6 +13,10 @@
 // alternate between even and odd tokens, so one workgroup barrier per token orders everything.
 // The state is read from its slot unless the sequence starts here (context length 0), and
 // written back at the end: a slot needs no clearing before it is used again.
+//
+// gla_scan_block_kernel (further down) is the same walk with 16 tokens per barrier, for runs of
+// rows; gla_piece_prefix_kernel / gla_combine_states_kernel join the pieces of a long run that
+// the layer walks at once (attention/recurrent.py).
 #include <atomic>
 #include <cstdlib>
 

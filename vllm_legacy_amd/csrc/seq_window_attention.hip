@@ -5,9 +5,13 @@
 // tensor serves both contractions (q . k_j reads rows, sum_j p_j k_j reads them again from L2 /
 // L1).  There is no value cache: a layer of this kind keeps half the bytes of an ordinary one.
 //
-// One kernel serves prompts, portions of prompts and decode steps: every query row reads its
+// Prompts, portions of prompts and decode steps are the same case: every query row reads its
 // window from the cache (the step's own keys are written first), so a position's result cannot
 // depend on how its sequence was cut into steps.  Scores, softmax and the weighted sum are fp32.
+// Four kernels, by dtype and by how the step's rows come: window_attention_kernel and
+// window_attention_group_kernel (any dtype, row by row), window_attention_heads_kernel (16-bit,
+// single rows on the matrix cores), window_attention_tile_kernel (16-bit, runs of rows on the
+// matrix cores); they differ by fp32 rounding.
 //
 // window_attention_kernel: one wave per (token, query head).  A tile is 64 keys: lane j computes
 // the score of key j against the query held in LDS (row reads of 16 bytes), the wave reduces
@@ -129,8 +133,8 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void window_attention_kernel
 // copies its tile into LDS with coalesced 16-byte loads (once, for all heads of the chunk), lane j
 // scores key j against every head's query, the probabilities go through LDS, every lane
 // accumulates two neighbouring dims of sum_j p_j k_j from the same tile, and the waves' (max, sum,
-// acc) are merged at the end.  The queries are read through wave-uniform addresses, so they sit
-// in scalar registers and the score loop's only LDS traffic is the key row.
+// acc) are merged at the end.  The queries are read through wave-uniform addresses (cache hits,
+// no LDS traffic): the score loop's only LDS traffic is the key row.
 constexpr int kHeadChunk = 4;
 constexpr int kPairs = kMaxDim / (2 * kWave);   // passes of 128 dims in the weighted sum
 
