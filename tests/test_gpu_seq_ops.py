@@ -376,14 +376,15 @@ def test_window_attention_batch_of_unequal_sequences():
 # ------------------------------------------------------------------------------ linear recurrence
 
 
+@pytest.mark.parametrize("n", [7, 45, 512, 530])       # few tokens: one thread per (token, channel); many: rows of W2 in registers
 @pytest.mark.parametrize("C,rank,dtype", [(8, 1, torch.float32), (96, 4, torch.float32), (300, 16, torch.float32),
-                                          (64, 8, torch.bfloat16)])
-def test_gla_log_decay(C, rank, dtype):
+                                          (64, 8, torch.bfloat16), (40, 32, torch.float32), (70, 33, torch.float32)])
+def test_gla_log_decay(C, rank, dtype, n):
     g = torch.Generator().manual_seed(C)
-    y = (torch.randn(7, rank + 2, generator=g) * 3).to(dtype).to(DEV)[:, 1:1 + rank]
+    y = (torch.randn(n, rank + 2, generator=g) * 3).to(dtype).to(DEV)[:, 1:1 + rank]
     w2 = torch.randn(C, rank, generator=g).to(dtype)
     bias = torch.randn(C, generator=g) * 4          # both tails of the sigmoid
-    out = torch.empty(7, C, dtype=torch.float32, device=DEV)
+    out = torch.empty(n, C, dtype=torch.float32, device=DEV)
     ops().gla_log_decay(out, y, w2.to(DEV), bias.to(DEV), 1 / 5.0)
     close(out, R.log_decay(y.cpu().to(R.F), w2.to(R.F), bias.to(R.F), 5.0), 1e-5)
     assert bool((out <= 0).all())

@@ -98,7 +98,7 @@ def run(args):
         x = model(ids_d, dec.positions, caches, dec)
         return model.compute_logits(x)
 
-    t = timed(lus_prefill, 5, 2)
+    t = timed(lus_prefill, 8, 6)
     e2e["lusadra_prefill_tokens_per_s"] = round(P / t, 1)
     t = timed(lus_decode, 20, 3)
     e2e["lusadra_decode_tokens_per_s"] = round(B / t, 1)
@@ -205,7 +205,7 @@ def run(args):
         hdn = llama(ids_d, pos_d, kv, meta_d)
         return llama.compute_logits(hdn)
 
-    t = timed(llama_prefill, 5, 2)
+    t = timed(llama_prefill, 8, 6)
     e2e["llama_prefill_tokens_per_s"] = round(P / t, 1)
     t = timed(llama_decode, 20, 3)
     e2e["llama_decode_tokens_per_s"] = round(B / t, 1)

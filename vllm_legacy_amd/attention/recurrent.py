@@ -49,6 +49,15 @@ class GatedLinearRecurrence(nn.Module):
         L = self.PIECE_ROWS
         if q is None or max(q) < 2 * L:
             return None
+        # the plan depends on the step and on where the scratch slots start, not on the layer:
+        # it is made (and copied to the device, in one transfer) once per step
+        cache = batch.__dict__.setdefault("_piece_plans", {})
+        key = (num_slots, L)
+        if key not in cache:
+            cache[key] = self._make_plan(q, c, sl, L, num_slots, batch.positions.device)
+        return cache[key]
+
+    def _make_plan(self, q, c, sl, L, num_slots, device):
         first_scratch = num_slots - self.SCRATCH_SLOTS
         starts, ctx, slots, cut, row, scratch = [0], [], [], [], 0, first_scratch
         for n, cb, sb in zip(q, c, sl):
@@ -67,7 +76,11 @@ class GatedLinearRecurrence(nn.Module):
                     starts.append(starts[-1] + min(L, n - i * L))
                 scratch += count
             row += n
-        return starts, ctx, slots, cut
+        # one int32 transfer: piece_start_loc | piece contexts | piece slots | 0 .. pieces - 1
+        flat = torch.tensor(starts + ctx + slots + list(range(len(ctx))), dtype=torch.int32).to(device)
+        n = len(ctx)
+        dev = (flat[:n + 1], flat[n + 1:2 * n + 1], flat[2 * n + 1:3 * n + 1], flat[3 * n + 1:])
+        return starts, ctx, slots, cut, dev
 
     def forward(self, out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                 gate: torch.Tensor, y: torch.Tensor, w2: torch.Tensor, bias: Optional[torch.Tensor],
@@ -89,25 +102,20 @@ class GatedLinearRecurrence(nn.Module):
         return out
 
     def _scan_in_pieces(self, o, q, k, v, log_decay, state, plan) -> None:
-        starts, ctx, slots, cut = plan
+        starts, ctx, slots, cut, (start_loc, ctx_dev, slots_dev, index_dev) = plan
         dev, L = q.device, self.PIECE_ROWS
         H, D, V = self.num_heads, self.head_dim, self.value_dim
-
-        def i32(x):
-            return torch.as_tensor(x, dtype=torch.int32).to(dev, non_blocking=True)
-
         for first, count, own, row, cb in cut:      # a continuing sequence starts from its state
             if cb > 0:
                 state[slots[first]].copy_(state[own])
-        start_loc = i32(starts)
-        ops.gla_scan(o, q, k, v, log_decay, state, start_loc, i32(ctx), i32(slots), self.q_scale,
+        ops.gla_scan(o, q, k, v, log_decay, state, start_loc, ctx_dev, slots_dev, self.q_scale,
                      max(b - a for a, b in zip(starts, starts[1:])))
         q_decayed = torch.empty((q.shape[0], H * D), dtype=torch.float32, device=dev)
         totals = torch.empty((len(ctx), H * D), dtype=torch.float32, device=dev)
         ops.gla_piece_prefix(q_decayed, totals, q, log_decay, start_loc, self.q_scale)
         for first, count, own, row, cb in cut:
             piece_slots = slots[first:first + count]
-            ops.gla_combine_states(state, i32(piece_slots), i32(list(range(first, first + count))), totals, own)
+            ops.gla_combine_states(state, slots_dev[first:first + count], index_dev[first:first + count], totals, own)
             n = starts[first + count] - starts[first]
             full = n // L                           # pieces of exactly L rows
             # pieces 1 .. full - 1 start from the states at the end of pieces 0 .. full - 2

@@ -33,6 +33,15 @@ std::atomic<int> g_scan_cols{[] {
   return v >= 0 && v <= 256 ? v : 0;
 }()};
 
+constexpr int kDecayTokens = 16;   // tokens a thread of the row-held form walks
+constexpr int kDecayRank = 32;     // widest projection whose row a thread holds in registers
+
+__device__ __forceinline__ float log_sigmoid_over_tau(float z, float inv_tau) {
+  // ln sigmoid(z) = -softplus(-z) = -(max(-z, 0) + log1p(exp(-|z|)))
+  return -(fmaxf(-z, 0.f) + log1pf(expf(-fabsf(z)))) * inv_tau;
+}
+
+// one thread per (token, channel): any rank
 template <class S>
 __global__ __launch_bounds__(256) void gla_log_decay_kernel(
     float* __restrict__ out, const typename S::T* __restrict__ y, int64_t y_stride,
@@ -45,9 +54,31 @@ __global__ __launch_bounds__(256) void gla_log_decay_kernel(
   const typename S::T* yr = y + (int64_t)t * y_stride;
   const typename S::T* wr = w2 + (int64_t)c * rank;
   for (int r = 0; r < rank; ++r) z += S::to_f32(wr[r]) * S::to_f32(yr[r]);
-  // softplus(-z) = max(-z, 0) + log1p(exp(-|z|))
-  const float sp = fmaxf(-z, 0.f) + log1pf(expf(-fabsf(z)));
-  out[(int64_t)t * channels + c] = -sp * inv_tau;
+  out[(int64_t)t * channels + c] = log_sigmoid_over_tau(z, inv_tau);
+}
+
+// rank <= kDecayRank: a thread keeps its channel's row of W2 in registers and walks
+// kDecayTokens tokens, whose y rows it reads through wave-uniform addresses
+template <class S>
+__global__ __launch_bounds__(256) void gla_log_decay_rows_kernel(
+    float* __restrict__ out, const typename S::T* __restrict__ y, int64_t y_stride,
+    const typename S::T* __restrict__ w2, const float* __restrict__ bias, float inv_tau,
+    int num_tokens, int channels, int rank) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= channels) return;
+  float w[kDecayRank];
+#pragma unroll
+  for (int r = 0; r < kDecayRank; ++r) w[r] = r < rank ? S::to_f32(w2[(int64_t)c * rank + r]) : 0.f;
+  const float b = bias != nullptr ? bias[c] : 0.f;
+  const int t0 = blockIdx.y * kDecayTokens, t1 = min(num_tokens, t0 + kDecayTokens);
+  for (int t = t0; t < t1; ++t) {
+    const typename S::T* yr = y + (int64_t)t * y_stride;
+    float z = b;
+#pragma unroll
+    for (int r = 0; r < kDecayRank; ++r)
+      if (r < rank) z += w[r] * S::to_f32(yr[r]);
+    out[(int64_t)t * channels + c] = log_sigmoid_over_tau(z, inv_tau);
+  }
 }
 
 template <class S, int ROWS>
@@ -372,10 +403,15 @@ extern "C" int vla_seq_gla_log_decay(float* out, const void* y, int64_t y_stride
     return VLA_ERR_ARG;
   return with_dtype(dtype, [&](auto s) {
     using S = decltype(s);
-    gla_log_decay_kernel<S><<<dim3((channels + 255) / 256, num_tokens), 256, 0,
-                              (hipStream_t)stream>>>(out, (const typename S::T*)y, y_stride,
-                                                     (const typename S::T*)w2, bias, inv_tau,
-                                                     channels, rank);
+    // (worth it once there are enough 16-token groups to fill the chip)
+    if (rank <= kDecayRank && num_tokens >= 32 * kDecayTokens)
+      gla_log_decay_rows_kernel<S><<<dim3((channels + 255) / 256, (num_tokens + kDecayTokens - 1) / kDecayTokens),
+                                     256, 0, (hipStream_t)stream>>>(
+          out, (const typename S::T*)y, y_stride, (const typename S::T*)w2, bias, inv_tau, num_tokens, channels,
+          rank);
+    else
+      gla_log_decay_kernel<S><<<dim3((channels + 255) / 256, num_tokens), 256, 0, (hipStream_t)stream>>>(
+          out, (const typename S::T*)y, y_stride, (const typename S::T*)w2, bias, inv_tau, channels, rank);
     VLA_SEQ_HIP_CHECK(hipGetLastError());
     return VLA_OK;
   });
