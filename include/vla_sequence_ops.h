@@ -126,6 +126,128 @@ int vla_seq_window_attention_tiles(void* out, int64_t out_stride, const void* q,
                                    int window, float scale, float temp_coef, float temp_every,
                                    float out_scale, int dtype, void* stream);
 
+/* ---- layers that norm a sublayer's input and its output -------------------------------------- */
+
+/* Activation codes of vla_seq_gated_act / vla_seq_grouped_linear. */
+#define VLA_ACT_NONE 0
+#define VLA_ACT_RELU 1
+#define VLA_ACT_RELU2 2      /* relu(z)^2 */
+#define VLA_ACT_SILU 3
+#define VLA_ACT_GELU_TANH 4  /* 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))) */
+
+/* One launch around a sublayer, on the fp32 stream x [T, width] (in place):
+ *   y given:        y' = y + y_bias (null: none);
+ *                   x += y' / sqrt(mean(y'^2) + eps) * post_weight * layer_scale (layer_scale null: 1)
+ *   add_row given:  x += add_row
+ *   out given:      out = out_dtype(x / sqrt(mean(x^2) + eps) * pre_weight)
+ * y is `y_dtype` rows of `width` values with stride y_stride; weights, layer_scale, add_row fp32
+ * [width].  All of it fp32. */
+int vla_seq_residual_norms(float* x, const void* y, int64_t y_stride, int y_dtype,
+                           const float* y_bias, const float* post_weight, const float* layer_scale,
+                           const float* add_row, void* out, const float* pre_weight, float eps,
+                           int num_tokens, int width, int out_dtype, void* stream);
+
+/* Causal convolution over time on each channel, added to its input:
+ *   out[t] = dtype(h[t] + sum_j weight[:, j] h[t - taps + 1 + j]),  zeros before a sequence's start,
+ * h fp32 [T, width], weight fp32 [width, taps].  The last taps - 1 inputs of a sequence live in
+ * state fp32 [num_slots, taps - 1, width] (oldest first): rows of earlier steps are read from
+ * there, and the step leaves its own last inputs there.  taps <= 16. */
+int vla_seq_causal_conv(void* out, const float* h, const float* weight, float* state,
+                        const int* query_start_loc, const int* context_lens,
+                        const int* state_slots, const int* token_seq, int num_tokens, int num_seqs,
+                        int num_slots, int width, int taps, int dtype, void* stream);
+
+/* out[t] = dtype([a[t]; b[t]]), a and b fp32 [T, width], out [T, 2 width]. */
+int vla_seq_concat_cast(void* out, const float* a, const float* b, int num_tokens, int width,
+                        int dtype, void* stream);
+
+/* out = act(gate) * up (up null: act(gate)); rows of `features` values with their own strides. */
+int vla_seq_gated_act(void* out, int64_t out_stride, const void* gate, int64_t gate_stride,
+                      const void* up, int64_t up_stride, int num_tokens, int features, int act,
+                      int dtype, void* stream);
+
+/* ---- attention over paged key and value caches with rotary positions ------------------------- */
+
+/* Rotates the step's queries in place and writes its rotated keys and values to the caches
+ * (keys [num_blocks, block_size, kv_heads, dim], values [.., kv_heads, vdim], `dtype`).  Pair i of
+ * the first rot_dims elements of a query / key head -- elements (2i, 2i + 1) when interleaved,
+ * (i, i + rot_dims / 2) otherwise -- turns by positions[t] * inv_freq[i]: (a, b) ->
+ * (a cos - b sin, b cos + a sin).  value_inv_freq [vdim / 2] (null: values are cached as they
+ * are) turns the pairs of a value head over all vdim elements the same way.  Angles are fp32
+ * products.  slot_mapping < 0 skips the caches. */
+int vla_seq_rotary_kv_write(void* q, int64_t q_stride, const void* k, int64_t k_stride,
+                            const void* v, int64_t v_stride, void* key_cache, void* value_cache,
+                            const int64_t* positions, const int64_t* slot_mapping,
+                            const float* inv_freq, const float* value_inv_freq, int num_tokens,
+                            int heads, int kv_heads, int dim, int vdim, int rot_dims,
+                            int interleaved, int block_size, int num_blocks, int dtype,
+                            void* stream);
+
+/* For the token at position p of sequence b and query head h (KV head h / (heads / kv_heads)):
+ *   s_j = (q . k_j) * scale  for max(0, p - window + 1) <= j <= p  (window <= 0: all j <= p)
+ *   o = sum_j softmax(s)_j v_j;  out_inv_freq given: pair m of o turns by -p * out_inv_freq[m]
+ *   out = dtype(o * sigmoid(gate[t, h]))                      (gate null: no gate)
+ * in fp32; the step's own keys and values must be in the caches already.  gate holds one number
+ * per (token, head) with row stride gate_stride. */
+int vla_seq_kv_attention(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                         const void* gate, int64_t gate_stride, const void* key_cache,
+                         const void* value_cache, const int* block_tables, int max_blocks,
+                         const int* token_seq, const int64_t* positions, const float* out_inv_freq,
+                         int interleaved, int num_tokens, int heads, int kv_heads, int dim, int vdim,
+                         int block_size, int num_blocks, int window, float scale, int dtype,
+                         void* stream);
+
+/* ---- element-wise gated recurrence (minGRU) ---------------------------------------------------- */
+
+/* S_t = (1 - z_t) S_(t-1) + z_t c_t per channel, z = sigmoid(zp), c = up + 1/2 where up >= 0 and
+ * sigmoid(up) below; out = dtype(S_t * silu(gp)).  zp, up, gp, out: `dtype` rows of `channels`
+ * values with their own strides; state fp32 [num_slots, channels]; a sequence with context 0
+ * starts from zero.  Runs of 256 rows and more are cut into pieces that are walked at once when
+ * scratch (fp32, vla_seq_mingru_scratch_floats values) is given. */
+int64_t vla_seq_mingru_scratch_floats(int num_seqs, int max_query_len, int channels);
+int vla_seq_mingru_scan(void* out, int64_t out_stride, const void* zp, int64_t z_stride,
+                        const void* up, int64_t u_stride, const void* gp, int64_t g_stride,
+                        float* state, const int* query_start_loc, const int* context_lens,
+                        const int* state_slots, int num_seqs, int num_slots, int max_query_len,
+                        int channels, float* scratch, int64_t scratch_floats, int dtype,
+                        void* stream);
+
+/* ---- mixture of experts in the activation dtype -------------------------------------------------- */
+
+/* Router of one token over `routed` experts (at most 512): z = router h in fp32 (router fp32
+ * [routed, width]), s = softmax(z), the `top` largest s + correction (null: s) are chosen, weights
+ * = their s / (sum + 1e-20).  experts int32 / weights fp32 [T, top].  shared_gate_weight fp32
+ * [width] (null: none): shared_gate[t] = sigmoid(shared_gate_weight . h). */
+int vla_seq_moe_route(const void* h, int64_t h_stride, const float* router,
+                      const float* correction, const float* shared_gate_weight, int* experts,
+                      float* weights, float* shared_gate, int num_tokens, int width, int routed,
+                      int top, int dtype, void* stream);
+
+/* Groups the pairs (token, choice) whose expert is below num_experts by expert, every group padded
+ * to whole tiles of vla_seq_moe_tile_rows() rows: pair_row int32 [T * top] (-1: the pair's expert
+ * has no weights), row_token int32 [max_tiles * tile rows] (-1: padding), tile_expert int32
+ * [max_tiles] (-1: unused).  max_tiles >= (T * top + (tile rows - 1) * min(num_experts, T * top))
+ * / tile rows, rounded up, holds every case. */
+int vla_seq_moe_tile_rows(void);
+int vla_seq_moe_plan(const int* experts, int num_tokens, int top, int num_experts, int* pair_row,
+                     int* row_token, int* tile_expert, int max_tiles, void* stream);
+
+/* out[row, :] = out_dtype(act(weight[e] a[src(row)])) for the rows of every tile, e =
+ * tile_expert[tile] (tiles with -1 are skipped), src(row) = row_token[row] (null: row; -1: a zero
+ * row).  weight `dtype` [experts, n_out, k_in], a `dtype` rows of k_in values. */
+int vla_seq_grouped_linear(void* out, int64_t out_stride, int out_dtype, const void* a,
+                           int64_t a_stride, const int* row_token, const void* weight,
+                           const int* tile_expert, int max_tiles, int n_out, int k_in, int act,
+                           int dtype, void* stream);
+
+/* out[t] (fp32 [T, width]) = sum_k weights[t, k] * (y[pair_row[t, k]] or, where pair_row is -1,
+ * h[t]) + shared_gate[t] * shared_y[t] (shared_y null: none; shared_gate null: 1).  y, shared_y
+ * fp32 rows of `width`. */
+int vla_seq_moe_combine(float* out, const float* y, const int* pair_row, const float* weights,
+                        const void* h, int64_t h_stride, const float* shared_y,
+                        const float* shared_gate, int num_tokens, int width, int top, int dtype,
+                        void* stream);
+
 /* Kernel choice for tests: window attention 0 = per shape, 1 = one wave per (row, head);
  * scan 0 = per shape, 1 = token by token. */
 int vla_seq_set_window_kernel(int mode);

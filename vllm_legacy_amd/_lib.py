@@ -55,6 +55,10 @@ SEQ_EXPORTS = [
     "vla_seq_gla_scan", "vla_seq_set_window_kernel", "vla_seq_window_attention_tiles",
     "vla_seq_window_attention_tiles_supported", "vla_seq_set_scan_kernel",
     "vla_seq_gla_piece_prefix", "vla_seq_gla_combine_states",
+    "vla_seq_residual_norms", "vla_seq_causal_conv", "vla_seq_concat_cast", "vla_seq_gated_act",
+    "vla_seq_rotary_kv_write", "vla_seq_kv_attention", "vla_seq_mingru_scratch_floats",
+    "vla_seq_mingru_scan", "vla_seq_moe_route", "vla_seq_moe_tile_rows", "vla_seq_moe_plan",
+    "vla_seq_grouped_linear", "vla_seq_moe_combine",
 ]
 _seq_lib = None
 
@@ -97,6 +101,23 @@ def seq_lib():
         L.vla_seq_gla_log_decay.argtypes = [p, p, i64, p, p, f, i, i, i, i, p]
         L.vla_seq_gla_scan.argtypes = [p, p, i64, p, i64, p, i64, p, p, p, p, p, f, i, i, i, i, i,
                                        i, i, p]
+        L.vla_seq_residual_norms.argtypes = [p, p, i64, i, p, p, p, p, p, p, f, i, i, i, p]
+        L.vla_seq_causal_conv.argtypes = [p, p, p, p, p, p, p, p, i, i, i, i, i, i, p]
+        L.vla_seq_concat_cast.argtypes = [p, p, p, i, i, i, p]
+        L.vla_seq_gated_act.argtypes = [p, i64, p, i64, p, i64, i, i, i, i, p]
+        L.vla_seq_rotary_kv_write.argtypes = [p, i64, p, i64, p, i64, p, p, p, p, p, p, i, i, i, i, i,
+                                              i, i, i, i, i, p]
+        L.vla_seq_kv_attention.argtypes = [p, i64, p, i64, p, i64, p, p, p, i, p, p, p, i, i, i, i, i,
+                                           i, i, i, i, f, i, p]
+        L.vla_seq_mingru_scratch_floats.argtypes = [i, i, i]
+        L.vla_seq_mingru_scratch_floats.restype = i64
+        L.vla_seq_mingru_scan.argtypes = [p, i64, p, i64, p, i64, p, i64, p, p, p, p, i, i, i, i, p,
+                                          i64, i, p]
+        L.vla_seq_moe_route.argtypes = [p, i64, p, p, p, p, p, p, i, i, i, i, i, p]
+        L.vla_seq_moe_tile_rows.argtypes = []
+        L.vla_seq_moe_plan.argtypes = [p, i, i, i, p, p, p, i, p]
+        L.vla_seq_grouped_linear.argtypes = [p, i64, i, p, i64, p, p, p, i, i, i, i, i, p]
+        L.vla_seq_moe_combine.argtypes = [p, p, p, p, p, i64, p, p, i, i, i, i, p]
         _seq_lib = L
     return _seq_lib
 

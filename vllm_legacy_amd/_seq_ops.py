@@ -255,3 +255,223 @@ def gla_combine_states(state: torch.Tensor, slots: torch.Tensor, pieces: torch.T
         seq_check(_lib.seq_lib().vla_seq_gla_combine_states(
             state.data_ptr(), slots.data_ptr(), pieces.data_ptr(), totals.data_ptr(), slots.numel(),
             int(final_slot), n, H, D, V, _stream(state.device)), "gla_combine_states")
+
+
+# ---------------------------------------------------------------- layers with norms on both sides
+ACT = {"none": 0, "relu": 1, "relu2": 2, "silu": 3, "gelu_tanh": 4}
+
+
+def residual_norms(x: torch.Tensor, y: Optional[torch.Tensor] = None, y_bias: Optional[torch.Tensor] = None,
+                   post_weight: Optional[torch.Tensor] = None,
+                   layer_scale: Optional[torch.Tensor] = None, add_row: Optional[torch.Tensor] = None,
+                   out: Optional[torch.Tensor] = None, pre_weight: Optional[torch.Tensor] = None,
+                   eps: float = 1e-5) -> None:
+    """x (fp32 [T, W], in place) += y' / rms(y') * post_weight * layer_scale with y' = y + y_bias;
+    x += add_row; out = x / rms(x) * pre_weight.  Each part is optional."""
+    _gpu(x, y, y_bias, post_weight, layer_scale, add_row, out, pre_weight)
+    T, W = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    for v in (y_bias, post_weight, layer_scale, add_row, pre_weight):
+        assert v is None or (v.dtype == torch.float32 and v.numel() == W and v.is_contiguous())
+    if y is not None:
+        assert y.shape == x.shape and post_weight is not None
+    if out is not None:
+        assert out.shape == x.shape and out.is_contiguous() and pre_weight is not None
+    with torch.cuda.device(x.device):
+        seq_check(_lib.seq_lib().vla_seq_residual_norms(
+            x.data_ptr(), _p(y), 0 if y is None else _rows(y, W), _lib.F32 if y is None else _dt(y.dtype),
+            _p(y_bias), _p(post_weight), _p(layer_scale), _p(add_row), _p(out), _p(pre_weight), float(eps), T, W,
+            _lib.F32 if out is None else _dt(out.dtype), _stream(x.device)), "residual_norms")
+
+
+def causal_conv(out: torch.Tensor, h: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tensor],
+                query_start_loc: torch.Tensor, context_lens: torch.Tensor, state_slots: torch.Tensor,
+                token_seq: torch.Tensor) -> None:
+    """out = h + conv(h) along time per channel; h fp32 [T, W]; weight fp32 [W, taps]; state fp32
+    [slots, taps - 1, W] holds every sequence's last inputs and is brought up to date."""
+    _gpu(out, h, weight, state, query_start_loc, context_lens, state_slots, token_seq)
+    T, W = h.shape
+    taps = weight.shape[1]
+    B = context_lens.numel()
+    assert h.dtype == torch.float32 and h.is_contiguous() and out.is_contiguous() and out.shape == h.shape
+    assert weight.dtype == torch.float32 and weight.is_contiguous() and weight.shape[0] == W
+    slots = 0
+    if taps > 1:
+        assert state is not None and state.dtype == torch.float32 and state.is_contiguous()
+        assert state.shape[1:] == (taps - 1, W)
+        slots = state.shape[0]
+    for t in (query_start_loc, context_lens, state_slots, token_seq):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    assert query_start_loc.numel() == B + 1 and state_slots.numel() == B and token_seq.numel() == T
+    with torch.cuda.device(h.device):
+        seq_check(_lib.seq_lib().vla_seq_causal_conv(
+            out.data_ptr(), h.data_ptr(), weight.data_ptr(), _p(state), query_start_loc.data_ptr(),
+            context_lens.data_ptr(), state_slots.data_ptr(), token_seq.data_ptr(), T, B, slots, W, taps,
+            _dt(out.dtype), _stream(h.device)), "causal_conv")
+
+
+def concat_cast(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor) -> None:
+    _gpu(out, a, b)
+    T, W = a.shape
+    assert a.dtype == b.dtype == torch.float32 and a.is_contiguous() and b.is_contiguous() and b.shape == a.shape
+    assert out.shape == (T, 2 * W) and out.is_contiguous()
+    with torch.cuda.device(a.device):
+        seq_check(_lib.seq_lib().vla_seq_concat_cast(out.data_ptr(), a.data_ptr(), b.data_ptr(), T, W,
+                                                     _dt(out.dtype), _stream(a.device)), "concat_cast")
+
+
+def gated_act(out: torch.Tensor, gate: torch.Tensor, up: Optional[torch.Tensor], act: str) -> None:
+    """out = act(gate) * up (up None: act(gate)); [T, F] views with free row strides."""
+    _gpu(out, gate, up)
+    T, F = gate.shape
+    assert out.shape == gate.shape and out.dtype == gate.dtype and (up is None or (up.shape == gate.shape and up.dtype == gate.dtype))
+    with torch.cuda.device(gate.device):
+        seq_check(_lib.seq_lib().vla_seq_gated_act(
+            out.data_ptr(), _rows(out, F), gate.data_ptr(), _rows(gate, F), _p(up),
+            0 if up is None else _rows(up, F), T, F, ACT[act], _dt(gate.dtype), _stream(gate.device)), "gated_act")
+
+
+def rotary_kv_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, key_cache: torch.Tensor,
+                    value_cache: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor,
+                    inv_freq: Optional[torch.Tensor], value_inv_freq: Optional[torch.Tensor], heads: int,
+                    rot_dims: int, interleaved: bool) -> None:
+    """q [T, H*D] rotated in place; k [T, G*D], v [T, G*V] rotated into the caches
+    [NB, BS, G, D] / [NB, BS, G, V]."""
+    _gpu(q, k, v, key_cache, value_cache, positions, slot_mapping, inv_freq, value_inv_freq)
+    NB, BS, G, D = key_cache.shape
+    V = value_cache.shape[3]
+    T = q.shape[0]
+    assert value_cache.shape[:3] == (NB, BS, G) and key_cache.is_contiguous() and value_cache.is_contiguous()
+    assert q.dtype == k.dtype == v.dtype == key_cache.dtype == value_cache.dtype
+    assert positions.dtype == torch.int64 and positions.numel() == T and positions.is_contiguous()
+    assert slot_mapping.dtype == torch.int64 and slot_mapping.numel() == T and slot_mapping.is_contiguous()
+    if rot_dims:
+        assert inv_freq.dtype == torch.float32 and inv_freq.numel() == rot_dims // 2 and inv_freq.is_contiguous()
+    if value_inv_freq is not None:
+        assert value_inv_freq.dtype == torch.float32 and value_inv_freq.numel() == V // 2
+    with torch.cuda.device(q.device):
+        seq_check(_lib.seq_lib().vla_seq_rotary_kv_write(
+            q.data_ptr(), _rows(q, heads * D), k.data_ptr(), _rows(k, G * D), v.data_ptr(), _rows(v, G * V),
+            key_cache.data_ptr(), value_cache.data_ptr(), positions.data_ptr(), slot_mapping.data_ptr(),
+            _p(inv_freq), _p(value_inv_freq), T, heads, G, D, V, int(rot_dims), int(bool(interleaved)), BS, NB,
+            _dt(q.dtype), _stream(q.device)), "rotary_kv_write")
+
+
+def kv_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tensor], key_cache: torch.Tensor,
+                 value_cache: torch.Tensor, block_tables: torch.Tensor, token_seq: torch.Tensor,
+                 positions: torch.Tensor, out_inv_freq: Optional[torch.Tensor], interleaved: bool, heads: int,
+                 window: int, scale: float) -> None:
+    """out [T, H*V] = softmax attention of q [T, H*D] over the caches, output pairs turned back by
+    the position, times sigmoid(gate [T, H])."""
+    _gpu(out, q, gate, key_cache, value_cache, block_tables, token_seq, positions, out_inv_freq)
+    NB, BS, G, D = key_cache.shape
+    V = value_cache.shape[3]
+    T = q.shape[0]
+    assert key_cache.is_contiguous() and value_cache.is_contiguous()
+    assert key_cache.dtype == value_cache.dtype == q.dtype == out.dtype
+    assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+    assert token_seq.dtype == torch.int32 and token_seq.numel() == T and token_seq.is_contiguous()
+    assert positions.dtype == torch.int64 and positions.numel() == T and positions.is_contiguous()
+    if out_inv_freq is not None:
+        assert out_inv_freq.dtype == torch.float32 and out_inv_freq.numel() == V // 2
+    if gate is not None:
+        assert gate.dtype == q.dtype
+    with torch.cuda.device(q.device):
+        seq_check(_lib.seq_lib().vla_seq_kv_attention(
+            out.data_ptr(), _rows(out, heads * V), q.data_ptr(), _rows(q, heads * D), _p(gate),
+            0 if gate is None else _rows(gate, heads), key_cache.data_ptr(), value_cache.data_ptr(),
+            block_tables.data_ptr(), block_tables.shape[1], token_seq.data_ptr(), positions.data_ptr(),
+            _p(out_inv_freq), int(bool(interleaved)), T, heads, G, D, V, BS, NB, int(window), float(scale),
+            _dt(q.dtype), _stream(q.device)), "kv_attention")
+
+
+def mingru_scan(out: torch.Tensor, zp: torch.Tensor, up: torch.Tensor, gp: torch.Tensor, state: torch.Tensor,
+                query_start_loc: torch.Tensor, context_lens: torch.Tensor, state_slots: torch.Tensor,
+                max_query_len: int) -> None:
+    """out, zp, up, gp: [T, R] views; state fp32 [slots, R]."""
+    _gpu(out, zp, up, gp, state, query_start_loc, context_lens, state_slots)
+    T, R = zp.shape
+    B = context_lens.numel()
+    assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1] == R
+    assert out.dtype == zp.dtype == up.dtype == gp.dtype
+    for t in (query_start_loc, context_lens, state_slots):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    L = _lib.seq_lib()
+    need = L.vla_seq_mingru_scratch_floats(B, int(max_query_len), R)
+    scratch = torch.empty(need, dtype=torch.float32, device=zp.device) if need else None
+    with torch.cuda.device(zp.device):
+        seq_check(L.vla_seq_mingru_scan(
+            out.data_ptr(), _rows(out, R), zp.data_ptr(), _rows(zp, R), up.data_ptr(), _rows(up, R),
+            gp.data_ptr(), _rows(gp, R), state.data_ptr(), query_start_loc.data_ptr(), context_lens.data_ptr(),
+            state_slots.data_ptr(), B, state.shape[0], int(max_query_len), R, _p(scratch), need, _dt(zp.dtype),
+            _stream(zp.device)), "mingru_scan")
+
+
+def moe_route(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor],
+              shared_gate_weight: Optional[torch.Tensor], top: int):
+    """-> experts int32 [T, top], weights fp32 [T, top], shared gate fp32 [T] or None."""
+    _gpu(h, router, correction, shared_gate_weight)
+    T, W = h.shape
+    N = router.shape[0]
+    assert router.dtype == torch.float32 and router.is_contiguous() and router.shape[1] == W
+    assert correction is None or (correction.dtype == torch.float32 and correction.numel() == N)
+    assert shared_gate_weight is None or (shared_gate_weight.dtype == torch.float32 and shared_gate_weight.numel() == W)
+    experts = torch.empty((T, top), dtype=torch.int32, device=h.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=h.device)
+    sg = None if shared_gate_weight is None else torch.empty((T, ), dtype=torch.float32, device=h.device)
+    with torch.cuda.device(h.device):
+        seq_check(_lib.seq_lib().vla_seq_moe_route(
+            h.data_ptr(), _rows(h, W), router.data_ptr(), _p(correction), _p(shared_gate_weight),
+            experts.data_ptr(), weights.data_ptr(), _p(sg), T, W, N, int(top), _dt(h.dtype), _stream(h.device)),
+            "moe_route")
+    return experts, weights, sg
+
+
+def moe_plan(experts: torch.Tensor, num_experts: int):
+    """-> pair_row int32 [T, top], row_token int32 [rows], tile_expert int32 [tiles]."""
+    _gpu(experts)
+    T, top = experts.shape
+    L = _lib.seq_lib()
+    tile = L.vla_seq_moe_tile_rows()
+    max_tiles = (T * top + (tile - 1) * min(num_experts, T * top) + tile - 1) // tile
+    pair_row = torch.empty((T, top), dtype=torch.int32, device=experts.device)
+    row_token = torch.empty((max_tiles * tile, ), dtype=torch.int32, device=experts.device)
+    tile_expert = torch.empty((max_tiles, ), dtype=torch.int32, device=experts.device)
+    assert experts.dtype == torch.int32 and experts.is_contiguous()
+    with torch.cuda.device(experts.device):
+        seq_check(L.vla_seq_moe_plan(experts.data_ptr(), T, top, int(num_experts), pair_row.data_ptr(),
+                                     row_token.data_ptr(), tile_expert.data_ptr(), max_tiles,
+                                     _stream(experts.device)), "moe_plan")
+    return pair_row, row_token, tile_expert
+
+
+def grouped_linear(out: torch.Tensor, a: torch.Tensor, row_token: Optional[torch.Tensor], weight: torch.Tensor,
+                   tile_expert: torch.Tensor, act: str = "none") -> None:
+    """out [tiles * tile rows, N] = act(weight[e] a[src(row)]); weight [E, N, K]; a rows of K."""
+    _gpu(out, a, row_token, weight, tile_expert)
+    E, N, K = weight.shape
+    assert weight.is_contiguous() and weight.dtype == a.dtype and a.shape[1] == K
+    L = _lib.seq_lib()
+    tiles = tile_expert.numel()
+    assert out.shape == (tiles * L.vla_seq_moe_tile_rows(), N) and out.is_contiguous()
+    assert row_token is None or (row_token.dtype == torch.int32 and row_token.numel() == out.shape[0])
+    if row_token is None:
+        assert a.shape[0] == out.shape[0]
+    with torch.cuda.device(a.device):
+        seq_check(L.vla_seq_grouped_linear(
+            out.data_ptr(), N, _dt(out.dtype), a.data_ptr(), _rows(a, K), _p(row_token), weight.data_ptr(),
+            tile_expert.data_ptr(), tiles, N, K, ACT[act], _dt(a.dtype), _stream(a.device)), "grouped_linear")
+
+
+def moe_combine(out: torch.Tensor, y: torch.Tensor, pair_row: torch.Tensor, weights: torch.Tensor,
+                h: torch.Tensor, shared_y: Optional[torch.Tensor], shared_gate: Optional[torch.Tensor]) -> None:
+    _gpu(out, y, pair_row, weights, h, shared_y, shared_gate)
+    T, W = h.shape
+    top = pair_row.shape[1]
+    assert out.dtype == torch.float32 and out.shape == (T, W) and out.is_contiguous()
+    assert y.dtype == torch.float32 and y.is_contiguous() and y.shape[1] == W
+    assert shared_y is None or (shared_y.dtype == torch.float32 and shared_y.is_contiguous() and shared_y.shape == (T, W))
+    with torch.cuda.device(h.device):
+        seq_check(_lib.seq_lib().vla_seq_moe_combine(
+            out.data_ptr(), y.data_ptr(), pair_row.data_ptr(), weights.data_ptr(), h.data_ptr(), _rows(h, W),
+            _p(shared_y), _p(shared_gate), T, W, top, _dt(h.dtype), _stream(h.device)), "moe_combine")

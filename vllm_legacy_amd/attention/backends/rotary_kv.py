@@ -1,0 +1,64 @@
+"""Causal softmax attention over paged key and value caches with rotary positions.
+
+The layer keeps two cache tensors, keys [num_blocks, block_size, kv_heads, dim] and values
+[num_blocks, block_size, kv_heads, vdim].  Queries and keys are rotated over their first `rot_dims`
+elements (pairs (2i, 2i + 1) when interleaved, (i, i + rot_dims / 2) otherwise, pair i by
+position * base^(-2i / rot_dims)).  With `rotate_values` the value of position j is rotated by j
+over all vdim elements before it is cached (pair m by j * base^(-2m / vdim)) and a head's output
+at position i is turned back by i, so that what a query reads of a value depends on their
+distance.  An optional window keeps 0 <= i - j < window; an optional gate multiplies each head's
+output by the sigmoid of one number per (token, head).  Every parameter is a constructor
+argument.  Prompts, portions of prompts and decode steps are one case: the step's keys and values
+are written to the caches, then every row reads from there (csrc/seq_kv_attention.hip).
+"""
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from vllm_legacy_amd import _seq_ops as ops
+from vllm_legacy_amd.attention.batch import SequenceBatch
+
+
+def inverse_frequencies(base: float, span: int, device=None) -> torch.Tensor:
+    """base^(-2i / span), i = 0 .. span / 2 - 1: formed in float64, rounded once to fp32."""
+    i = torch.arange(span // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / float(span))
+    return f.to(torch.float32).to(device)
+
+
+class RotaryKVAttention(nn.Module):
+
+    def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float,
+                 rot_dims: int, rot_base: float, interleaved: bool = True, rotate_values: bool = False,
+                 window: Optional[int] = None, device=None) -> None:
+        super().__init__()
+        assert num_heads % num_kv_heads == 0 and 0 <= rot_dims <= head_dim and rot_dims % 2 == 0
+        assert not rotate_values or value_dim % 2 == 0
+        self.num_heads, self.num_kv_heads = num_heads, num_kv_heads
+        self.head_dim, self.value_dim = head_dim, value_dim
+        self.scale, self.rot_dims, self.interleaved = float(scale), int(rot_dims), bool(interleaved)
+        self.window = int(window) if window else 0
+        self.register_buffer("inv_freq", inverse_frequencies(rot_base, rot_dims, device) if rot_dims else None,
+                             persistent=False)
+        self.register_buffer("value_inv_freq",
+                             inverse_frequencies(rot_base, value_dim, device) if rotate_values else None,
+                             persistent=False)
+
+    @staticmethod
+    def get_cache_shapes(num_blocks: int, block_size: int, num_kv_heads: int, head_dim: int,
+                         value_dim: int) -> Tuple[Tuple[int, ...], Tuple[int, ...]]:
+        return ((num_blocks, block_size, num_kv_heads, head_dim),
+                (num_blocks, block_size, num_kv_heads, value_dim))
+
+    def forward(self, out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                gate: Optional[torch.Tensor], key_cache: torch.Tensor, value_cache: torch.Tensor,
+                batch: SequenceBatch) -> torch.Tensor:
+        """q [T, H * D] (rotated in place), k [T, G * D], v [T, G * V], gate [T, H], out [T, H * V]:
+        views with free row strides."""
+        ops.rotary_kv_write(q, k, v, key_cache, value_cache, batch.positions, batch.slot_mapping,
+                            self.inv_freq, self.value_inv_freq, self.num_heads, self.rot_dims, self.interleaved)
+        ops.kv_attention(out, q, gate, key_cache, value_cache, batch.block_tables, batch.token_seq,
+                         batch.positions, self.value_inv_freq, self.interleaved, self.num_heads, self.window,
+                         self.scale)
+        return out

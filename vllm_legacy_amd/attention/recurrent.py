@@ -128,3 +128,26 @@ class GatedLinearRecurrence(nn.Module):
                 r0 = row + full * L
                 qd = q_decayed[r0:row + n].view(n - full * L, H, D).permute(1, 0, 2)    # [H, l, D]
                 o[r0:row + n].permute(1, 0, 2).add_(torch.matmul(qd, state[piece_slots[full - 1]]))
+
+
+class MinGRURecurrence(nn.Module):
+    """Element-wise gated recurrence whose gates read only the current token:
+    S_t = (1 - z_t) S_(t-1) + z_t c_t with z = sigmoid(zp) and the candidate c = up + 1/2 where
+    up >= 0, sigmoid(up) below; the output is S_t * silu(gp).  zp, up, gp are projections of the
+    token (biases included).  One fp32 number per channel and sequence lives in a state slot
+    [num_slots, channels]; a sequence whose context length is 0 starts from zero.  Long runs of
+    rows are walked in pieces at the same time (csrc/seq_gated_recurrence.hip)."""
+
+    def __init__(self, channels: int) -> None:
+        super().__init__()
+        self.channels = channels
+
+    @staticmethod
+    def get_state_shape(num_slots: int, channels: int) -> Tuple[int, ...]:
+        return (num_slots, channels)
+
+    def forward(self, out: torch.Tensor, zp: torch.Tensor, up: torch.Tensor, gp: torch.Tensor,
+                state: torch.Tensor, batch: SequenceBatch) -> torch.Tensor:
+        ops.mingru_scan(out, zp, up, gp, state, batch.query_start_loc, batch.context_lens, batch.state_slots,
+                        batch.max_query_len)
+        return out

@@ -137,3 +137,43 @@ class SinusoidalEmbedding(nn.Module):
                           device=self.weight.device)
         seq_ops.embed_positions(out, self.weight.data, input_ids, positions, self.inv_freq)
         return out
+
+
+class CausalConvMix(nn.Module):
+    """h + conv(h): a causal convolution over time on each channel (weight [width, taps], no bias,
+    tap j reads the input taps - 1 - j tokens back), added to its input.  The last taps - 1 inputs
+    of every sequence live in a state slot [num_slots, taps - 1, width] (fp32), so a sequence may be
+    cut anywhere.  Reads the fp32 rows a norm left and writes the activation dtype."""
+
+    def __init__(self, width: int, taps: int, device=None):
+        super().__init__()
+        self.taps = int(taps)
+        self.weight = nn.Parameter(torch.zeros((width, taps), dtype=torch.float32, device=device),
+                                   requires_grad=False)
+
+    @staticmethod
+    def get_state_shape(num_slots: int, width: int, taps: int) -> Tuple[int, ...]:
+        return (num_slots, max(taps - 1, 0), width)
+
+    def forward(self, h: torch.Tensor, state: Optional[torch.Tensor], batch, out_dtype: torch.dtype) -> torch.Tensor:
+        out = torch.empty(h.shape, dtype=out_dtype, device=h.device)
+        seq_ops.causal_conv(out, h, self.weight.data, state if self.taps > 1 else None, batch.query_start_loc,
+                            batch.context_lens, batch.state_slots, batch.token_seq)
+        return out
+
+
+class GatedActivation(nn.Module):
+    """act(gate) * up on the two halves of a merged projection [T, 2 F] (gate | up), or act(z) on
+    a plain one; act: relu, relu2 (the square of relu), silu, gelu_tanh."""
+
+    def __init__(self, act: str, gated: bool = True):
+        super().__init__()
+        if act not in seq_ops.ACT or act == "none":
+            raise ValueError(f"unknown activation {act!r}")
+        self.act, self.gated = act, gated
+
+    def forward(self, z: torch.Tensor) -> torch.Tensor:
+        F = z.shape[1] // 2 if self.gated else z.shape[1]
+        out = torch.empty((z.shape[0], F), dtype=z.dtype, device=z.device)
+        seq_ops.gated_act(out, z[:, :F], z[:, F:] if self.gated else None, self.act)
+        return out

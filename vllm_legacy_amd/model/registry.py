@@ -11,6 +11,7 @@ import torch
 # architecture -> (module, model class, config class)
 _MODELS: Dict[str, Tuple[str, str, str]] = {
     "Lusadra": ("vllm_legacy_amd.model.lusadra", "LusadraForCausalLM", "LusadraConfig"),
+    "Dopipel": ("vllm_legacy_amd.model.dopipel", "DopipelForCausalLM", "DopipelConfig"),
     # the synthetic-weight Llama stack behind the engine's model protocol
     "LlamaDecodeStack": ("vllm_legacy_amd.engine.llama_adapter", "PagedLlamaForEngine", "LlamaEngineConfig"),
 }

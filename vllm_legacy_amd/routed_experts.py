@@ -1,0 +1,99 @@
+"""Mixture-of-experts feed-forward in the activation dtype, routed on the device.
+
+Router: z = W_r h in fp32 over all routed experts, s = softmax(z); the `top` experts with the
+largest s + correction are chosen and weighted by their s renormalized to sum 1.  The last
+`identity` routed experts have no weights: their output is the token's input.  An expert is
+W_down act(W_up h).  An optional shared expert of the same form runs for every token, multiplied by
+sigmoid(w_sg . h).  The output is fp32 (the caller norms it and adds it to its stream).
+
+Execution (csrc/seq_moe_kernels.hip): route -> plan (pairs grouped by expert into row tiles) ->
+grouped up-projection with the activation fused (rows gathered from the tokens) -> grouped
+down-projection in fp32 -> combine (weighted sum per token in the order of its choices, identity
+experts and the shared expert added there).  Nothing synchronises with the host.
+"""
+from typing import Dict, Optional
+
+import torch
+import torch.nn as nn
+
+from vllm_legacy_amd import _seq_ops as ops
+
+
+def mm_f32(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """a [T, K] x w [N, K]^T with an fp32 result (16-bit operands keep the fp32 accumulator)."""
+    if a.dtype == torch.float32:
+        return torch.mm(a, w.t())
+    return torch.mm(a, w.t(), out_dtype=torch.float32)
+
+
+class RoutedExperts(nn.Module):
+
+    def __init__(self, width: int, num_experts: int, num_identity: int, top: int, expert_ff: int,
+                 shared_ff: int = 0, act: str = "relu2", shared_act: Optional[str] = None,
+                 dtype=torch.bfloat16, device=None) -> None:
+        super().__init__()
+        if top > num_experts + num_identity:
+            raise ValueError("top exceeds the number of routed experts")
+        self.width, self.num_experts, self.num_identity, self.top = width, num_experts, num_identity, top
+        self.expert_ff, self.shared_ff, self.act = expert_ff, shared_ff, act
+        self.shared_act = shared_act or act
+        self.dtype = dtype
+        routed = num_experts + num_identity
+
+        def par(shape, dt):
+            return nn.Parameter(torch.zeros(shape, dtype=dt, device=device), requires_grad=False)
+
+        self.router = par((routed, width), torch.float32)
+        self.correction = par((routed, ), torch.float32)
+        self.w_up = par((num_experts, expert_ff, width), dtype)
+        self.w_down = par((num_experts, width, expert_ff), dtype)
+        if shared_ff:
+            self.shared_up = par((shared_ff, width), dtype)
+            self.shared_down = par((width, shared_ff), dtype)
+            self.shared_gate = par((width, ), torch.float32)
+
+    def set_weights(self, t: Dict[str, torch.Tensor]) -> None:
+        """t: router, correction (optional), e<i>.up / e<i>.down, shared.up / shared.down / shared.sg."""
+        dev, dt = self.router.device, self.dtype
+        routed = self.num_experts + self.num_identity
+
+        def put(param, value, name):
+            if tuple(value.shape) != tuple(param.shape):
+                raise ValueError(f"{name}: shape {tuple(value.shape)}, expected {tuple(param.shape)}")
+            param.data = value.to(param.dtype).to(dev).contiguous()
+
+        put(self.router, t["router"], "router")
+        if "correction" in t:
+            put(self.correction, t["correction"].reshape(routed), "correction")
+        if self.num_experts:
+            put(self.w_up, torch.stack([t[f"e{e}.up"] for e in range(self.num_experts)]).to(dt), "e*.up")
+            put(self.w_down, torch.stack([t[f"e{e}.down"] for e in range(self.num_experts)]).to(dt), "e*.down")
+        if self.shared_ff:
+            put(self.shared_up, t["shared.up"], "shared.up")
+            put(self.shared_down, t["shared.down"], "shared.down")
+            put(self.shared_gate, t["shared.sg"].reshape(self.width), "shared.sg")
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        """h [T, width] in the activation dtype -> fp32 [T, width]."""
+        T = h.shape[0]
+        experts, weights, sg = ops.moe_route(h, self.router.data, self.correction.data,
+                                             self.shared_gate.data if self.shared_ff else None, self.top)
+        if self.num_experts:
+            pair_row, row_token, tile_expert = ops.moe_plan(experts, self.num_experts)
+            rows = row_token.numel()
+            u = torch.empty((rows, self.expert_ff), dtype=h.dtype, device=h.device)
+            ops.grouped_linear(u, h, row_token, self.w_up.data, tile_expert, self.act)
+            y = torch.empty((rows, self.width), dtype=torch.float32, device=h.device)
+            ops.grouped_linear(y, u, None, self.w_down.data, tile_expert)
+        else:   # identity experts only
+            pair_row = torch.full((T, self.top), -1, dtype=torch.int32, device=h.device)
+            y = torch.zeros((1, self.width), dtype=torch.float32, device=h.device)
+        shared_y = None
+        if self.shared_ff:
+            su = torch.mm(h, self.shared_up.data.t())
+            sa = torch.empty_like(su)
+            ops.gated_act(sa, su, None, self.shared_act)
+            shared_y = mm_f32(sa, self.shared_down.data)
+        out = torch.empty((T, self.width), dtype=torch.float32, device=h.device)
+        ops.moe_combine(out, y, pair_row, weights, h, shared_y, sg)
+        return out
