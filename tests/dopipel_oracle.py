@@ -57,46 +57,58 @@ def rotate_pairs(u, angle, layout="interleaved"):
     return out
 
 
+def attention_core(q, k, v, gate_logits, spec, window=0):
+    """q [n, H, D], k [n, G, D], v [n, G, V] before any rotation, gate_logits [n, H] or None, of one
+    sequence from its first token.  Returns [n, H, V] after the gate."""
+    n = q.shape[0]
+    H, G, V = spec["heads"], spec["kv_heads"], spec["vdim"]
+    rot = spec["rot"]
+    layout = rot.get("layout", "interleaved")
+    pos = torch.arange(n)
+    if rot["dims"]:
+        ang = pair_angles(pos, rot["dims"] // 2, rot["base"], rot["dims"])
+        q, k = rotate_pairs(q, ang, layout), rotate_pairs(k, ang, layout)
+    vang = pair_angles(pos, V // 2, rot["base"], V)
+    v = rotate_pairs(v, vang, layout)
+    out = torch.zeros(n, H, V, dtype=F)
+    for a in range(n):
+        lo = max(0, a - window + 1) if window else 0
+        for hh in range(H):
+            g = hh // (H // G)
+            s = (k[lo:a + 1, g] @ q[a, hh]) * spec["scale"]
+            out[a, hh] = torch.softmax(s, 0) @ v[lo:a + 1, g]
+    out = rotate_pairs(out, -vang, layout)
+    if gate_logits is not None:
+        out = out * torch.sigmoid(gate_logits)[:, :, None]
+    return out
+
+
 def rotary_attention(h, t, spec):
     """The attention mixer on its input h [n, width]; t: this layer's mixer tensors by short name."""
     n = h.shape[0]
     H, G, D, V = spec["heads"], spec["kv_heads"], spec["dim"], spec["vdim"]
-    rot = spec["rot"]
-    layout = rot.get("layout", "interleaved")
-    pos = torch.arange(n)
     q = (h @ t["q"].T + t["q.b"]).view(n, H, D)
     k = (h @ t["k"].T + t["k.b"]).view(n, G, D)
     v = (h @ t["v"].T + t["v.b"]).view(n, G, V)
-    ang = pair_angles(pos, rot["dims"] // 2, rot["base"], rot["dims"])
-    q, k = rotate_pairs(q, ang, layout), rotate_pairs(k, ang, layout)
-    vang = pair_angles(pos, V // 2, rot["base"], V)
-    v = rotate_pairs(v, vang, layout)
-    gate = torch.sigmoid(h @ t["g"].T)                      # [n, H]
-    out = torch.zeros(n, H, V, dtype=F)
-    for a in range(n):
-        for hh in range(H):
-            g = hh // (H // G)
-            s = (k[:a + 1, g] @ q[a, hh]) * spec["scale"]
-            p = torch.softmax(s, 0)
-            out[a, hh] = p @ v[:a + 1, g]
-    out = rotate_pairs(out, -vang, layout) * gate[:, :, None]
+    out = attention_core(q, k, v, h @ t["g"].T, spec)
     return out.reshape(n, H * V) @ t["o"].T + t["o.b"]
+
+
+def mingru_core(zp, up, gp):
+    """Pre-activations [n, R] of one sequence from its first token -> gated outputs [n, R]."""
+    z = torch.sigmoid(zp)
+    cand = torch.where(up >= 0, up + 0.5, torch.sigmoid(up))
+    S = torch.zeros(zp.shape[1], dtype=F)
+    out = torch.zeros_like(zp)
+    for i in range(zp.shape[0]):
+        S = (1 - z[i]) * S + z[i] * cand[i]
+        out[i] = S * gp[i] * torch.sigmoid(gp[i])
+    return out
 
 
 def mingru(h, t):
     """Gated recurrence whose gates read only the current token."""
-    n = h.shape[0]
-    z = torch.sigmoid(h @ t["z"].T + t["z.b"])
-    u = h @ t["x"].T + t["x.b"]
-    cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
-    gate = h @ t["g"].T
-    gate = gate * torch.sigmoid(gate)
-    S = torch.zeros(z.shape[1], dtype=F)
-    out = torch.zeros_like(z)
-    for i in range(n):
-        S = (1 - z[i]) * S + z[i] * cand[i]
-        out[i] = S * gate[i]
-    return out @ t["o"].T
+    return mingru_core(h @ t["z"].T + t["z.b"], h @ t["x"].T + t["x.b"], h @ t["g"].T) @ t["o"].T
 
 
 def dense_ff(h, t):
@@ -140,7 +152,8 @@ def layer(x, i, cfg, W):
     spec, eps = cfg["layers"][i], cfg["norm"]["eps"]
     t = sub(W, f"l{i}.")
     h = rms_norm(x, t["norm1"], eps)
-    h = input_convolution(h, t["canon1"])
+    if "canon1" in t:
+        h = input_convolution(h, t["canon1"])
     if spec["type"] == "attention":
         y = rotary_attention(h, sub(t, "mix."), spec["mixer"])
     elif spec["type"] == "mingru":
