@@ -197,6 +197,23 @@ int vla_seq_kv_attention(void* out, int64_t out_stride, const void* q, int64_t q
                          int block_size, int num_blocks, int window, float scale, int dtype,
                          void* stream);
 
+/* The same attention for 16-bit activations, tiled over runs of 32 query rows of a sequence on
+ * the matrix cores: rows query_start_loc[b] .. query_start_loc[b + 1] - 1 of sequence b sit at
+ * positions context_lens[b] ...  dim and vdim must be multiples of 32, at most 128
+ * (vla_seq_kv_attention_tiles_supported); query rows and cache rows must be 8-byte aligned.
+ * vla_seq_kv_attention takes single rows of such shapes to the matrix cores by itself;
+ * vla_seq_set_kv_attention_kernel(1) keeps both off them (tests run both), 0 is the default. */
+int vla_seq_kv_attention_tiles_supported(int dim, int vdim, int dtype);
+int vla_seq_kv_attention_tiles(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                               const void* gate, int64_t gate_stride, const void* key_cache,
+                               const void* value_cache, const int* block_tables, int max_blocks,
+                               const int* query_start_loc, const int* context_lens,
+                               const float* out_inv_freq, int interleaved, int num_seqs,
+                               int max_query_len, int heads, int kv_heads, int dim, int vdim,
+                               int block_size, int num_blocks, int window, float scale, int dtype,
+                               void* stream);
+int vla_seq_set_kv_attention_kernel(int mode);
+
 /* ---- element-wise gated recurrence (minGRU) ---------------------------------------------------- */
 
 /* S_t = (1 - z_t) S_(t-1) + z_t c_t per channel, z = sigmoid(zp), c = up + 1/2 where up >= 0 and

@@ -234,6 +234,7 @@ ATTN_SHAPES = [
     (2, 1, 96, 96, 96, "interleaved"),
     (8, 1, 64, 32, 32, "halves"),
     (5, 5, 128, 128, 64, "interleaved"),
+    (2, 1, 32, 96, 32, "halves"),
 ]
 
 
@@ -251,6 +252,23 @@ def test_rotary_attention_prompt_portions_and_decoding(shape, dtype):
     for cuts in ([n], [2, 3, 4, 5, 1, 7, 2] * 5, [40] + [1] * 35, [33, 35, 7], [1] * n):
         got = run_attention(spec, q, k, v, gate, cuts, dtype)
         assert float((got - want).abs().max()) <= bar * float(want.abs().max()), (cuts[:3], float((got - want).abs().max()))
+
+
+def test_plain_and_matrix_core_kernels_agree():
+    """bfloat16 through the kernel every dtype can take and through the matrix-core kernels."""
+    from vllm_legacy_amd import _seq_ops as ops
+    H, G, D, V = 6, 2, 96, 64
+    spec = attention_spec(H, G, D, V, 64, 1000.0)
+    n = 101
+    q, k, v, gate = (t.to(torch.bfloat16).float() for t in (rnd((n, H, D), 0), rnd((n, G, D), 1), rnd((n, G, V), 2), rnd((n, H), 3)))
+    fast = run_attention(spec, q, k, v, gate, [60, 3] + [1] * 38, torch.bfloat16)
+    ops.set_kv_attention_kernel(1)
+    try:
+        plain = run_attention(spec, q, k, v, gate, [60, 3] + [1] * 38, torch.bfloat16)
+    finally:
+        ops.set_kv_attention_kernel(0)
+    assert float((fast - plain).abs().max()) <= 0.03 * float(plain.abs().max())
+    assert not torch.equal(fast, plain)          # two kernels did run
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -385,6 +385,45 @@ def kv_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tensor
             _dt(q.dtype), _stream(q.device)), "kv_attention")
 
 
+def set_kv_attention_kernel(mode: int) -> None:
+    """0: kv_attention picks its kernel per shape; 1: never the matrix-core kernels."""
+    seq_check(_lib.seq_lib().vla_seq_set_kv_attention_kernel(mode), "set_kv_attention_kernel")
+
+
+def kv_attention_tiles_supported(q: torch.Tensor, head_dim: int, value_dim: int) -> bool:
+    """Whether the matrix-core kernel for runs of query rows takes this query tensor."""
+    return bool(_lib.seq_lib().vla_seq_kv_attention_tiles_supported(head_dim, value_dim, _dt(q.dtype))) and \
+        q.data_ptr() % 8 == 0 and (q.stride(0) * q.element_size()) % 8 == 0
+
+
+def kv_attention_tiles(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tensor], key_cache: torch.Tensor,
+                       value_cache: torch.Tensor, block_tables: torch.Tensor, query_start_loc: torch.Tensor,
+                       context_lens: torch.Tensor, max_query_len: int, out_inv_freq: Optional[torch.Tensor],
+                       interleaved: bool, heads: int, window: int, scale: float) -> None:
+    """The same attention as kv_attention for 16-bit activations, tiled over runs of 32 query rows
+    of a sequence."""
+    _gpu(out, q, gate, key_cache, value_cache, block_tables, query_start_loc, context_lens, out_inv_freq)
+    NB, BS, G, D = key_cache.shape
+    V = value_cache.shape[3]
+    B = context_lens.numel()
+    assert key_cache.is_contiguous() and value_cache.is_contiguous()
+    assert key_cache.dtype == value_cache.dtype == q.dtype == out.dtype
+    for t in (block_tables, query_start_loc, context_lens):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    assert block_tables.dim() == 2 and block_tables.shape[0] == B and query_start_loc.numel() == B + 1
+    if out_inv_freq is not None:
+        assert out_inv_freq.dtype == torch.float32 and out_inv_freq.numel() == V // 2
+    if gate is not None:
+        assert gate.dtype == q.dtype
+    with torch.cuda.device(q.device):
+        seq_check(_lib.seq_lib().vla_seq_kv_attention_tiles(
+            out.data_ptr(), _rows(out, heads * V), q.data_ptr(), _rows(q, heads * D), _p(gate),
+            0 if gate is None else _rows(gate, heads), key_cache.data_ptr(), value_cache.data_ptr(),
+            block_tables.data_ptr(), block_tables.shape[1], query_start_loc.data_ptr(), context_lens.data_ptr(),
+            _p(out_inv_freq), int(bool(interleaved)), B, int(max_query_len), heads, G, D, V, BS, NB, int(window),
+            float(scale), _dt(q.dtype), _stream(q.device)), "kv_attention_tiles")
+
+
 def mingru_scan(out: torch.Tensor, zp: torch.Tensor, up: torch.Tensor, gp: torch.Tensor, state: torch.Tensor,
                 query_start_loc: torch.Tensor, context_lens: torch.Tensor, state_slots: torch.Tensor,
                 max_query_len: int) -> None:

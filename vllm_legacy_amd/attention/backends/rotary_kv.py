@@ -9,7 +9,10 @@ at position i is turned back by i, so that what a query reads of a value depends
 distance.  An optional window keeps 0 <= i - j < window; an optional gate multiplies each head's
 output by the sigmoid of one number per (token, head).  Every parameter is a constructor
 argument.  Prompts, portions of prompts and decode steps are one case: the step's keys and values
-are written to the caches, then every row reads from there (csrc/seq_kv_attention.hip).
+are written to the caches, then every row reads from there (csrc/seq_kv_attention.hip: matrix-core
+kernels for 16-bit models whose head sizes are multiples of 32 -- tiles of 32 rows for runs of
+rows, all heads of a KV group at once for single rows -- and an fp32 kernel for any dtype and head
+size).
 """
 from typing import Optional, Tuple
 
@@ -28,6 +31,8 @@ def inverse_frequencies(base: float, span: int, device=None) -> torch.Tensor:
 
 
 class RotaryKVAttention(nn.Module):
+    # steps whose longest run of rows is at least this long take the tiled kernel (16-bit models)
+    TILE_MIN_QUERY = 4
 
     def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float,
                  rot_dims: int, rot_base: float, interleaved: bool = True, rotate_values: bool = False,
@@ -58,7 +63,14 @@ class RotaryKVAttention(nn.Module):
         views with free row strides."""
         ops.rotary_kv_write(q, k, v, key_cache, value_cache, batch.positions, batch.slot_mapping,
                             self.inv_freq, self.value_inv_freq, self.num_heads, self.rot_dims, self.interleaved)
-        ops.kv_attention(out, q, gate, key_cache, value_cache, batch.block_tables, batch.token_seq,
-                         batch.positions, self.value_inv_freq, self.interleaved, self.num_heads, self.window,
-                         self.scale)
+        if batch.max_query_len >= self.TILE_MIN_QUERY and \
+                ops.kv_attention_tiles_supported(q, self.head_dim, self.value_dim):
+            # a step with runs of rows (prompts, portions): 32-row tiles on the matrix cores
+            ops.kv_attention_tiles(out, q, gate, key_cache, value_cache, batch.block_tables,
+                                   batch.query_start_loc, batch.context_lens, batch.max_query_len,
+                                   self.value_inv_freq, self.interleaved, self.num_heads, self.window, self.scale)
+        else:
+            ops.kv_attention(out, q, gate, key_cache, value_cache, batch.block_tables, batch.token_seq,
+                             batch.positions, self.value_inv_freq, self.interleaved, self.num_heads, self.window,
+                             self.scale)
         return out

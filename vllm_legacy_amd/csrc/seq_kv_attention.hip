@@ -217,6 +217,537 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void kv_attention_kernel(
                        out_inv_freq, interleaved, gv, lane, kWave);
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Matrix-core kernels for 16-bit models.  Both products run in transposed form on 32x32x8 MFMAs,
+// lane = (hf, c) = (lane >> 5, lane & 31):
+//   S^T = K q^T   A = K    lane: key c, dims 8 ks + 4 hf .. + 3
+//                 B = q^T  lane: query c, the same dims (registers, loaded once)
+//                 C        lane: query c, keys (i & 3) + 8 (i >> 2) + 4 hf, i = 0 .. 15
+//   O^T = V^T P^T A = V^T  lane: value dim 32 n + c, keys 8 s + 4 hf .. + 3
+//                 B = P^T  lane: query c, the same keys = registers 4 s .. 4 s + 3 of C above
+//                 C        lane: query c, dims 32 n + (i & 3) + 8 (i >> 2) + 4 hf
+// so a lane owns one query's scores, running max / sum and output column, and both elements of
+// every rotated output pair (neighbours when interleaved; vdim / 2 = 16 (vdim / 32) apart
+// otherwise, which moves n and i >> 2 but neither hf nor c).  Scores leave the first product in
+// fp32 and stay there; a weight enters the second product as the sum of two 16-bit numbers (its
+// rounding and the rounding of what the rounding lost).
+template <class S>
+struct Mfma8;
+template <>
+struct Mfma8<BF16> {
+  typedef short V4 __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ f32x16 run(u32x2 a, u32x2 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(V4, a), __builtin_bit_cast(V4, b), c,
+                                                    0, 0, 0);
+  }
+};
+template <>
+struct Mfma8<F16> {
+  typedef _Float16 V4 __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ f32x16 run(u32x2 a, u32x2 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(V4, a), __builtin_bit_cast(V4, b), c, 0,
+                                                0, 0);
+  }
+};
+template <class S>
+__device__ __forceinline__ uint32_t bits16(float v) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, S::from_f32(v));
+}
+template <class S>
+__device__ __forceinline__ float from_bits16(uint32_t b) {
+  return S::to_f32(__builtin_bit_cast(typename S::T, (uint16_t)b));
+}
+
+constexpr int kTile = 32;
+std::atomic<int> g_kv_kernel{0};
+
+// dim index of register i of output block n for lane half hf
+__device__ __forceinline__ constexpr int out_dim(int n, int i, int hf) {
+  return 32 * n + (i & 3) + 8 * (i >> 2) + 4 * hf;
+}
+
+// Turns the output pairs a lane holds back by the query's position (o[n][i] normalized already).
+template <int VB>
+__device__ __forceinline__ void turn_back(f32x16 (&o)[VB], int hf, float p,
+                                          const float* __restrict__ out_inv_freq, int interleaved) {
+  constexpr int VD = 32 * VB;
+  if (interleaved) {
+#pragma unroll
+    for (int n = 0; n < VB; ++n)
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        float s, c;
+        sincosf(p * out_inv_freq[out_dim(n, i, hf) >> 1], &s, &c);
+        const float a = o[n][i], b = o[n][i + 1];
+        o[n][i] = a * c + b * s;
+        o[n][i + 1] = b * c - a * s;
+      }
+  } else {
+    // partner of dim d < VD / 2 is d + 16 VB: block n + VB / 2 (and, for odd VB, i + 8)
+#pragma unroll
+    for (int n = 0; n < VB; ++n)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int d = 32 * n + (i & 3) + 8 * (i >> 2);      // without 4 hf: same for both halves
+        if (d < VD / 2) {
+          const int d2 = d + VD / 2;
+          const int n2 = d2 / 32, r2 = d2 % 32;
+          const int i2 = (r2 & 3) + 4 * (r2 >> 3);
+          float s, c;
+          sincosf(p * out_inv_freq[d + 4 * hf], &s, &c);
+          const float a = o[n][i], b = o[n2][i2];
+          o[n][i] = a * c + b * s;
+          o[n2][i2] = b * c - a * s;
+        }
+      }
+  }
+}
+
+// kv_attention_tile_kernel<S, DB, VB>: runs of rows (prompts, portions).  One workgroup per
+// (sequence, tile of 32 consecutive query rows, KV head, chunk of up to four of its query heads);
+// wave w takes query head w of the chunk.  The keys and values from the first row's window start
+// to the last row walk through LDS in tiles of 32, staged once for all waves: keys row-major for
+// the first product, values transposed for the second.
+template <class S, int DB, int VB>
+__global__ __launch_bounds__(256) void kv_attention_tile_kernel(
+    typename S::T* __restrict__ out, int64_t out_stride, const typename S::T* __restrict__ q,
+    int64_t q_stride, const typename S::T* __restrict__ gate, int64_t gate_stride,
+    const typename S::T* __restrict__ key_cache, const typename S::T* __restrict__ value_cache,
+    const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ query_start_loc,
+    const int* __restrict__ context_lens, const float* __restrict__ out_inv_freq, int interleaved,
+    int heads, int kv_heads, int block_size, int num_blocks, int window, float scale) {
+  using T = typename S::T;
+  using M = Mfma8<S>;
+  constexpr int D = 32 * DB, VD = 32 * VB;
+  constexpr int KROW = D + 4, TROW = kTile + 4;      // elements; both keep 8-byte alignment
+  __shared__ __align__(16) T k_lds[kTile * KROW];    // [key][dim]
+  __shared__ __align__(16) T vt_lds[VD * TROW];      // [value dim][key]
+  const int b = blockIdx.z;
+  const int t0 = query_start_loc[b] + kTile * blockIdx.x;
+  const int nq = min(kTile, query_start_loc[b + 1] - t0);
+  if (nq <= 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int hf = lane >> 5, c = lane & 31;
+  const int group = heads / kv_heads;
+  const int chunks = (group + 3) / 4;
+  const int g = blockIdx.y / chunks;
+  const int h = g * group + (blockIdx.y % chunks) * 4 + w;
+  const bool active = h < g * group + group;
+  const int p0 = context_lens[b] + kTile * blockIdx.x, p_last = p0 + nq - 1;
+  const int j_lo = window > 0 ? max(0, p0 - window + 1) : 0;
+  const int* table = block_tables + (int64_t)b * max_blocks;
+  const int pq = p0 + c;
+
+  u32x2 qf[D / 8];
+#pragma unroll
+  for (int ks = 0; ks < D / 8; ++ks) {
+    u32x2 v = {0u, 0u};
+    if (active && c < nq)
+      v = *reinterpret_cast<const u32x2*>(q + (int64_t)(t0 + c) * q_stride + (int64_t)h * D + 8 * ks + 4 * hf);
+    qf[ks] = v;
+  }
+  f32x16 o[VB];
+#pragma unroll
+  for (int n = 0; n < VB; ++n)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[n][i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  // staging: DB + VB pieces of 8 bytes per thread and tile, loaded one tile ahead
+  u32x2 xk[DB], xv[VB];
+  auto fetch = [&](int j0) {
+    auto token = [&](int j) {
+      int blk = table[j / block_size];
+      blk = (unsigned)blk < (unsigned)num_blocks ? blk : 0;
+      return ((long long)blk * block_size + j % block_size) * kv_heads + g;
+    };
+#pragma unroll
+    for (int u = 0; u < DB; ++u) {
+      const int i = tid + 256 * u;
+      const int r = i / (D / 4), v = i % (D / 4);
+      const int j = j0 + r;
+      const long long off = j <= p_last ? token(j) * D + 4 * v : 0;
+      const u32x2 got = *reinterpret_cast<const u32x2*>(key_cache + off);
+      xk[u] = j <= p_last ? got : u32x2{0u, 0u};
+    }
+#pragma unroll
+    for (int u = 0; u < VB; ++u) {
+      const int i = tid + 256 * u;
+      const int r = i / (VD / 4), v = i % (VD / 4);
+      const int j = j0 + r;
+      const long long off = j <= p_last ? token(j) * VD + 4 * v : 0;
+      const u32x2 got = *reinterpret_cast<const u32x2*>(value_cache + off);
+      xv[u] = j <= p_last ? got : u32x2{0u, 0u};
+    }
+  };
+  fetch(j_lo);
+  for (int j0 = j_lo; j0 <= p_last; j0 += kTile) {
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < DB; ++u) {
+      const int i = tid + 256 * u;
+      const int r = i / (D / 4), v = i % (D / 4);
+      *reinterpret_cast<u32x2*>(k_lds + r * KROW + 4 * v) = xk[u];
+    }
+#pragma unroll
+    for (int u = 0; u < VB; ++u) {
+      const int i = tid + 256 * u;
+      const int r = i / (VD / 4), v = i % (VD / 4);
+      uint16_t* col = reinterpret_cast<uint16_t*>(vt_lds) + (4 * v) * TROW + r;
+      col[0] = (uint16_t)(xv[u][0] & 0xffffu);
+      col[TROW] = (uint16_t)(xv[u][0] >> 16);
+      col[2 * TROW] = (uint16_t)(xv[u][1] & 0xffffu);
+      col[3 * TROW] = (uint16_t)(xv[u][1] >> 16);
+    }
+    if (j0 + kTile <= p_last) fetch(j0 + kTile);
+    __syncthreads();
+    if (!active) continue;
+    f32x16 st;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) st[i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < D / 8; ++ks) {
+      const u32x2 a = *reinterpret_cast<const u32x2*>(k_lds + c * KROW + 8 * ks + 4 * hf);
+      st = M::run(a, qf[ks], st);
+    }
+    float mt = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int key = j0 + (i & 3) + 8 * (i >> 2) + 4 * hf;
+      const int dist = pq - key;
+      const bool ok = c < nq && dist >= 0 && (window <= 0 || dist < window);
+      st[i] = ok ? st[i] * scale : -INFINITY;
+      mt = fmaxf(mt, st[i]);
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(m, mt);
+    const float corr = m_new == -INFINITY ? 1.f : expf(m - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      st[i] = m_new == -INFINITY ? 0.f : expf(st[i] - m_new);
+      psum += st[i];
+    }
+    l = l * corr + psum;          // this lane's keys; the partner's half is added at the end
+    m = m_new;
+#pragma unroll
+    for (int n = 0; n < VB; ++n)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[n][i] *= corr;
+#pragma unroll
+    for (int s8 = 0; s8 < 4; ++s8) {
+      uint32_t hb[4], lb[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float pv = st[4 * s8 + e];
+        hb[e] = bits16<S>(pv);
+        lb[e] = bits16<S>(pv - from_bits16<S>(hb[e]));
+      }
+      const u32x2 hi = {hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16)};
+      const u32x2 lo = {lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16)};
+#pragma unroll
+      for (int n = 0; n < VB; ++n) {
+        const u32x2 a = *reinterpret_cast<const u32x2*>(vt_lds + (32 * n + c) * TROW + 8 * s8 + 4 * hf);
+        o[n] = M::run(a, hi, o[n]);
+        o[n] = M::run(a, lo, o[n]);
+      }
+    }
+  }
+  if (!active) return;
+  l += __shfl_xor(l, 32, 64);
+  if (c >= nq) return;
+  const float inv = 1.f / l;
+#pragma unroll
+  for (int n = 0; n < VB; ++n)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[n][i] *= inv;
+  if (out_inv_freq != nullptr) turn_back<VB>(o, hf, (float)pq, out_inv_freq, interleaved);
+  float gv = 1.f;
+  if (gate != nullptr) gv = 1.f / (1.f + expf(-S::to_f32(gate[(int64_t)(t0 + c) * gate_stride + h])));
+#pragma unroll
+  for (int n = 0; n < VB; ++n)
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      out[(int64_t)(t0 + c) * out_stride + (int64_t)h * VD + out_dim(n, i, hf)] = S::from_f32(o[n][i] * gv);
+}
+
+// kv_attention_heads_kernel<S, DB, VB>: single rows (decode steps).  One workgroup per (row, KV
+// head, chunk of up to 32 of its query heads): the 32 columns of the products hold the chunk's
+// query heads, so each key and value byte is read once per KV head whatever the group size.  The
+// kRowWaves waves split the window's tiles (wave w takes tiles w, w + kRowWaves, ...), each with
+// its own key and value tiles in LDS and its own running max / sum / output, merged at the end.
+constexpr int kRowWaves = 8;
+
+template <class S, int DB, int VB>
+__global__ __launch_bounds__(64 * kRowWaves) void kv_attention_heads_kernel(
+    typename S::T* __restrict__ out, int64_t out_stride, const typename S::T* __restrict__ q,
+    int64_t q_stride, const typename S::T* __restrict__ gate, int64_t gate_stride,
+    const typename S::T* __restrict__ key_cache, const typename S::T* __restrict__ value_cache,
+    const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ token_seq,
+    const int64_t* __restrict__ positions, const float* __restrict__ out_inv_freq, int interleaved,
+    int heads, int kv_heads, int block_size, int num_blocks, int window, float scale,
+    int merge_heads) {
+  using T = typename S::T;
+  using M = Mfma8<S>;
+  constexpr int D = 32 * DB, VD = 32 * VB;
+  constexpr int KROW = D + 4, VROW = VD + 4;
+  constexpr int WAVE_ELEMS = kTile * (KROW + VROW);       // one wave's two tiles, in elements
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int hf = lane >> 5, c = lane & 31;
+  T* k_lds = reinterpret_cast<T*>(smem) + (size_t)w * WAVE_ELEMS;
+  T* v_lds = k_lds + kTile * KROW;
+  const int t = blockIdx.x;
+  const int group = heads / kv_heads;
+  const int chunks = (group + 31) / 32;
+  const int g = blockIdx.y / chunks;
+  const int h0 = g * group + (blockIdx.y % chunks) * 32;
+  const int nh = min(32, g * group + group - h0);
+  const int p = (int)positions[t];
+  const int* table = block_tables + (int64_t)token_seq[t] * max_blocks;
+  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const bool live = c < nh;
+  u32x2 qf[D / 8];
+#pragma unroll
+  for (int ks = 0; ks < D / 8; ++ks) {
+    u32x2 v = {0u, 0u};
+    if (live)
+      v = *reinterpret_cast<const u32x2*>(q + (int64_t)t * q_stride + (int64_t)(h0 + c) * D + 8 * ks + 4 * hf);
+    qf[ks] = v;
+  }
+  f32x16 o[VB];
+#pragma unroll
+  for (int n = 0; n < VB; ++n)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[n][i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  // A wave's share of a tile is D / 8 + VD / 8 pieces of 8 bytes per lane, all issued before any
+  // is used and one tile ahead.  Lanes 0..31 look the 32 tokens of the tile up once and hand the
+  // row numbers round with shuffles.
+  constexpr int KP = D / 8, VP = VD / 8;
+  u32x2 xk[KP], xv[VP];
+  auto fetch = [&](int j0) {
+    const int jr = j0 + c;
+    long long row = -1;
+    if (jr <= p) {
+      int blk = table[jr / block_size];
+      blk = (unsigned)blk < (unsigned)num_blocks ? blk : 0;
+      row = ((long long)blk * block_size + jr % block_size) * kv_heads + g;
+    }
+#pragma unroll
+    for (int u = 0; u < KP; ++u) {
+      const int i = lane + kWave * u;
+      const int r = i / (D / 4), v = i % (D / 4);
+      const long long rb = __shfl(row, r, 64);
+      const u32x2 got = *reinterpret_cast<const u32x2*>(key_cache + (rb >= 0 ? rb * D + 4 * v : 0));
+      xk[u] = rb >= 0 ? got : u32x2{0u, 0u};
+    }
+#pragma unroll
+    for (int u = 0; u < VP; ++u) {
+      const int i = lane + kWave * u;
+      const int r = i / (VD / 4), v = i % (VD / 4);
+      const long long rb = __shfl(row, r, 64);
+      const u32x2 got = *reinterpret_cast<const u32x2*>(value_cache + (rb >= 0 ? rb * VD + 4 * v : 0));
+      xv[u] = rb >= 0 ? got : u32x2{0u, 0u};
+    }
+  };
+  fetch(lo + w * kTile);
+  for (int j0 = lo + w * kTile; j0 <= p; j0 += kRowWaves * kTile) {
+#pragma unroll
+    for (int u = 0; u < KP; ++u) {
+      const int i = lane + kWave * u;
+      const int r = i / (D / 4), v = i % (D / 4);
+      *reinterpret_cast<u32x2*>(k_lds + r * KROW + 4 * v) = xk[u];
+    }
+#pragma unroll
+    for (int u = 0; u < VP; ++u) {
+      const int i = lane + kWave * u;
+      const int r = i / (VD / 4), v = i % (VD / 4);
+      *reinterpret_cast<u32x2*>(v_lds + r * VROW + 4 * v) = xv[u];
+    }
+    if (j0 + kRowWaves * kTile <= p) fetch(j0 + kRowWaves * kTile);
+    wave_sync();
+    f32x16 st;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) st[i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < D / 8; ++ks) {
+      const u32x2 a = *reinterpret_cast<const u32x2*>(k_lds + c * KROW + 8 * ks + 4 * hf);
+      st = M::run(a, qf[ks], st);
+    }
+    float mt = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int dist = p - (j0 + (i & 3) + 8 * (i >> 2) + 4 * hf);
+      st[i] = (live && dist >= 0) ? st[i] * scale : -INFINITY;
+      mt = fmaxf(mt, st[i]);
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(m, mt);
+    const float corr = m_new == -INFINITY ? 1.f : expf(m - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      st[i] = m_new == -INFINITY ? 0.f : expf(st[i] - m_new);
+      psum += st[i];
+    }
+    l = l * corr + psum;
+    m = m_new;
+#pragma unroll
+    for (int n = 0; n < VB; ++n)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[n][i] *= corr;
+#pragma unroll
+    for (int s8 = 0; s8 < 4; ++s8) {
+      uint32_t hb[4], lb[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float pv = st[4 * s8 + e];
+        hb[e] = bits16<S>(pv);
+        lb[e] = bits16<S>(pv - from_bits16<S>(hb[e]));
+      }
+      const u32x2 hi = {hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16)};
+      const u32x2 lo2 = {lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16)};
+#pragma unroll
+      for (int n = 0; n < VB; ++n) {
+        // V^T operand from the row-major tile: value dim 32 n + c of keys 8 s8 + 4 hf .. + 3
+        const uint16_t* col = reinterpret_cast<const uint16_t*>(v_lds) + (8 * s8 + 4 * hf) * VROW + 32 * n + c;
+        const u32x2 a = {(uint32_t)col[0] | ((uint32_t)col[VROW] << 16),
+                         (uint32_t)col[2 * VROW] | ((uint32_t)col[3 * VROW] << 16)};
+        o[n] = M::run(a, hi, o[n]);
+        o[n] = M::run(a, lo2, o[n]);
+      }
+    }
+    wave_sync();
+  }
+  l += __shfl_xor(l, 32, 64);
+  // merge the waves through LDS (the tiles are done with): [wave][head][2 + VD]
+  __syncthreads();
+  float* merge = reinterpret_cast<float*>(smem);
+  if (live) {
+    float* mine = merge + ((size_t)w * merge_heads + c) * (2 + VD);
+    if (hf == 0) {
+      mine[0] = m;
+      mine[1] = l;
+    }
+#pragma unroll
+    for (int n = 0; n < VB; ++n)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mine[2 + out_dim(n, i, hf)] = o[n][i];
+  }
+  __syncthreads();
+  auto merged = [&](int hh, int d) {
+    float mm = -INFINITY;
+    for (int ww = 0; ww < kRowWaves; ++ww) mm = fmaxf(mm, merge[((size_t)ww * merge_heads + hh) * (2 + VD)]);
+    float ll = 0.f, ov = 0.f;
+    for (int ww = 0; ww < kRowWaves; ++ww) {
+      const float* src = merge + ((size_t)ww * merge_heads + hh) * (2 + VD);
+      const float f = src[0] == -INFINITY ? 0.f : expf(src[0] - mm);
+      ll += src[1] * f;
+      ov += src[2 + d] * f;
+    }
+    return ov / ll;
+  };
+  for (int i = tid; i < nh * VD; i += 64 * kRowWaves) {
+    const int hh = i / VD, d = i - hh * VD;
+    float val = merged(hh, d);
+    if (out_inv_freq != nullptr) {
+      const bool is_a = interleaved ? (d & 1) == 0 : d < VD / 2;
+      const int other = interleaved ? (d ^ 1) : (is_a ? d + VD / 2 : d - VD / 2);
+      const int f = interleaved ? d >> 1 : (is_a ? d : d - VD / 2);
+      float s, c2;
+      sincosf((float)p * out_inv_freq[f], &s, &c2);
+      const float ov = merged(hh, other);
+      val = is_a ? val * c2 + ov * s : val * c2 - ov * s;
+    }
+    if (gate != nullptr) val *= 1.f / (1.f + expf(-S::to_f32(gate[(int64_t)t * gate_stride + h0 + hh])));
+    out[(int64_t)t * out_stride + (int64_t)(h0 + hh) * VD + d] = S::from_f32(val);
+  }
+}
+
+template <class S, int DB, int VB>
+int launch_heads_one(dim3 grid, hipStream_t stream, typename S::T* out, int64_t out_stride,
+                     const typename S::T* q, int64_t q_stride, const typename S::T* gate,
+                     int64_t gate_stride, const typename S::T* key_cache,
+                     const typename S::T* value_cache, const int* block_tables, int max_blocks,
+                     const int* token_seq, const int64_t* positions, const float* out_inv_freq,
+                     int interleaved, int heads, int kv_heads, int block_size, int num_blocks,
+                     int window, float scale) {
+  constexpr int D = 32 * DB, VD = 32 * VB;
+  const int group = heads / kv_heads;
+  const int merge_heads = group < 32 ? group : 32;
+  const size_t tiles = (size_t)kRowWaves * kTile * (D + 4 + VD + 4) * sizeof(typename S::T);
+  const size_t merge = (size_t)kRowWaves * merge_heads * (2 + VD) * sizeof(float);
+  const size_t lds = tiles > merge ? tiles : merge;
+  if (lds > 160 * 1024) return VLA_ERR_HEAD_SIZE;
+  static std::atomic<size_t> allowed{64 * 1024};   // raised once per kernel, not per launch
+  if (lds > allowed.load(std::memory_order_relaxed)) {
+    VLA_SEQ_HIP_CHECK(hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&kv_attention_heads_kernel<S, DB, VB>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    allowed.store(lds, std::memory_order_relaxed);
+  }
+  kv_attention_heads_kernel<S, DB, VB><<<grid, 64 * kRowWaves, lds, stream>>>(
+      out, out_stride, q, q_stride, gate, gate_stride, key_cache, value_cache, block_tables,
+      max_blocks, token_seq, positions, out_inv_freq, interleaved, heads, kv_heads, block_size,
+      num_blocks, window, scale, merge_heads);
+  VLA_SEQ_HIP_CHECK(hipGetLastError());
+  return VLA_OK;
+}
+
+template <class S, int DB, int VB>
+int launch_tiles_one(dim3 grid, hipStream_t stream, typename S::T* out, int64_t out_stride,
+                     const typename S::T* q, int64_t q_stride, const typename S::T* gate,
+                     int64_t gate_stride, const typename S::T* key_cache,
+                     const typename S::T* value_cache, const int* block_tables, int max_blocks,
+                     const int* qsl, const int* ctx, const float* out_inv_freq, int interleaved,
+                     int heads, int kv_heads, int block_size, int num_blocks, int window,
+                     float scale) {
+  kv_attention_tile_kernel<S, DB, VB><<<grid, 256, 0, stream>>>(
+      out, out_stride, q, q_stride, gate, gate_stride, key_cache, value_cache, block_tables,
+      max_blocks, qsl, ctx, out_inv_freq, interleaved, heads, kv_heads, block_size, num_blocks,
+      window, scale);
+  VLA_SEQ_HIP_CHECK(hipGetLastError());
+  return VLA_OK;
+}
+
+// dim / 32 and vdim / 32 in 1 .. 4 -> the instantiation
+#define VLA_KV_BY_SIZE(FN, S, db, vb, ...)                         \
+  switch ((db) * 4 + (vb)-5) {                                     \
+    case 0: return FN<S, 1, 1>(__VA_ARGS__);                       \
+    case 1: return FN<S, 1, 2>(__VA_ARGS__);                       \
+    case 2: return FN<S, 1, 3>(__VA_ARGS__);                       \
+    case 3: return FN<S, 1, 4>(__VA_ARGS__);                       \
+    case 4: return FN<S, 2, 1>(__VA_ARGS__);                       \
+    case 5: return FN<S, 2, 2>(__VA_ARGS__);                       \
+    case 6: return FN<S, 2, 3>(__VA_ARGS__);                       \
+    case 7: return FN<S, 2, 4>(__VA_ARGS__);                       \
+    case 8: return FN<S, 3, 1>(__VA_ARGS__);                       \
+    case 9: return FN<S, 3, 2>(__VA_ARGS__);                       \
+    case 10: return FN<S, 3, 3>(__VA_ARGS__);                      \
+    case 11: return FN<S, 3, 4>(__VA_ARGS__);                      \
+    case 12: return FN<S, 4, 1>(__VA_ARGS__);                      \
+    case 13: return FN<S, 4, 2>(__VA_ARGS__);                      \
+    case 14: return FN<S, 4, 3>(__VA_ARGS__);                      \
+    case 15: return FN<S, 4, 4>(__VA_ARGS__);                      \
+    default: return VLA_ERR_HEAD_SIZE;                             \
+  }
+
+template <class S, class... A>
+int launch_heads(int db, int vb, A... a) {
+  VLA_KV_BY_SIZE(launch_heads_one, S, db, vb, a...)
+}
+template <class S, class... A>
+int launch_tiles(int db, int vb, A... a) {
+  VLA_KV_BY_SIZE(launch_tiles_one, S, db, vb, a...)
+}
+
+bool mfma_sizes(int dim, int vdim) {
+  return dim % 32 == 0 && dim >= 32 && dim <= 128 && vdim % 32 == 0 && vdim >= 32 && vdim <= 128;
+}
+
 }  // namespace
 }  // namespace seq
 }  // namespace vla
@@ -269,6 +800,21 @@ extern "C" int vla_seq_kv_attention(void* out, int64_t out_stride, const void* q
   return with_dtype(dtype, [&](auto s) {
     using S = decltype(s);
     using T = typename S::T;
+    if constexpr (sizeof(T) == 2) {
+      // 16-bit rows on the matrix cores when the head sizes and the alignment allow
+      if (g_kv_kernel.load(std::memory_order_relaxed) == 0 && mfma_sizes(dim, vdim) &&
+          ((uintptr_t)q % 8) == 0 && ((q_stride * 2) % 8) == 0 && ((uintptr_t)key_cache % 8) == 0 &&
+          ((uintptr_t)value_cache % 8) == 0) {
+        const int group = heads / kv_heads;
+        const dim3 grid(num_tokens, kv_heads * ((group + 31) / 32));
+        const int rc = launch_heads<S>(dim / 32, vdim / 32, grid, (hipStream_t)stream, (T*)out, out_stride,
+                                       (const T*)q, q_stride, (const T*)gate, gate_stride,
+                                       (const T*)key_cache, (const T*)value_cache, block_tables,
+                                       max_blocks, token_seq, positions, out_inv_freq, interleaved,
+                                       heads, kv_heads, block_size, num_blocks, window, scale);
+        if (rc != VLA_ERR_HEAD_SIZE) return rc;
+      }
+    }
     const dim3 grid(num_tokens, (heads + kHeadsPerGroup - 1) / kHeadsPerGroup);
     kv_attention_kernel<S><<<grid, kWave * kHeadsPerGroup, 0, (hipStream_t)stream>>>(
         (T*)out, out_stride, (const T*)q, q_stride, (const T*)gate, gate_stride,
@@ -277,4 +823,49 @@ extern "C" int vla_seq_kv_attention(void* out, int64_t out_stride, const void* q
     VLA_SEQ_HIP_CHECK(hipGetLastError());
     return VLA_OK;
   });
+}
+
+// 0: pick per shape; 1: always the one-wave-per-(row, head) kernel (tests run both)
+extern "C" int vla_seq_set_kv_attention_kernel(int mode) {
+  if (mode < 0 || mode > 1) return VLA_ERR_ARG;
+  g_kv_kernel.store(mode, std::memory_order_relaxed);
+  return VLA_OK;
+}
+
+extern "C" int vla_seq_kv_attention_tiles_supported(int dim, int vdim, int dtype) {
+  return (dtype == VLA_F16 || dtype == VLA_BF16) && mfma_sizes(dim, vdim) &&
+         g_kv_kernel.load(std::memory_order_relaxed) == 0;
+}
+
+extern "C" int vla_seq_kv_attention_tiles(
+    void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* gate,
+    int64_t gate_stride, const void* key_cache, const void* value_cache, const int* block_tables,
+    int max_blocks, const int* query_start_loc, const int* context_lens, const float* out_inv_freq,
+    int interleaved, int num_seqs, int max_query_len, int heads, int kv_heads, int dim, int vdim,
+    int block_size, int num_blocks, int window, float scale, int dtype, void* stream) {
+  if (num_seqs == 0 || max_query_len == 0) return VLA_OK;
+  if (!out || !q || !key_cache || !value_cache || !block_tables || !query_start_loc || !context_lens ||
+      num_seqs < 0 || num_seqs > 65535 || max_query_len < 0 || heads <= 0 || kv_heads <= 0 ||
+      heads % kv_heads != 0 || block_size <= 0 || num_blocks <= 0 || max_blocks <= 0 ||
+      out_stride < (int64_t)heads * vdim || q_stride < (int64_t)heads * dim ||
+      (gate && gate_stride < heads))
+    return VLA_ERR_ARG;
+  if ((dtype != VLA_F16 && dtype != VLA_BF16) || !mfma_sizes(dim, vdim)) return VLA_ERR_HEAD_SIZE;
+  // 8-byte fragment loads: query rows and cache rows must allow them
+  if (((uintptr_t)q % 8) || ((q_stride * 2) % 8) || ((uintptr_t)key_cache % 8) ||
+      ((uintptr_t)value_cache % 8))
+    return VLA_ERR_ARG;
+  const int group = heads / kv_heads;
+  const dim3 grid((max_query_len + kTile - 1) / kTile, kv_heads * ((group + 3) / 4), num_seqs);
+  if (dtype == VLA_BF16)
+    return launch_tiles<BF16>(dim / 32, vdim / 32, grid, (hipStream_t)stream, (__bf16*)out, out_stride,
+                              (const __bf16*)q, q_stride, (const __bf16*)gate, gate_stride,
+                              (const __bf16*)key_cache, (const __bf16*)value_cache, block_tables,
+                              max_blocks, query_start_loc, context_lens, out_inv_freq, interleaved,
+                              heads, kv_heads, block_size, num_blocks, window, scale);
+  return launch_tiles<F16>(dim / 32, vdim / 32, grid, (hipStream_t)stream, (_Float16*)out, out_stride,
+                           (const _Float16*)q, q_stride, (const _Float16*)gate, gate_stride,
+                           (const _Float16*)key_cache, (const _Float16*)value_cache, block_tables,
+                           max_blocks, query_start_loc, context_lens, out_inv_freq, interleaved, heads,
+                           kv_heads, block_size, num_blocks, window, scale);
 }
