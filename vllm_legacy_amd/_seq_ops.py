@@ -393,7 +393,7 @@ def set_kv_attention_kernel(mode: int) -> None:
 def kv_attention_tiles_supported(q: torch.Tensor, head_dim: int, value_dim: int) -> bool:
     """Whether the matrix-core kernel for runs of query rows takes this query tensor."""
     return bool(_lib.seq_lib().vla_seq_kv_attention_tiles_supported(head_dim, value_dim, _dt(q.dtype))) and \
-        q.data_ptr() % 8 == 0 and (q.stride(0) * q.element_size()) % 8 == 0
+        q.data_ptr() % 16 == 0 and (q.stride(0) * q.element_size()) % 16 == 0
 
 
 def kv_attention_tiles(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tensor], key_cache: torch.Tensor,

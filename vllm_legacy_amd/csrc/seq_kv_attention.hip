@@ -304,11 +304,43 @@ __device__ __forceinline__ void turn_back(f32x16 (&o)[VB], int hf, float p,
   }
 }
 
-// kv_attention_tile_kernel<S, DB, VB>: runs of rows (prompts, portions).  One workgroup per
-// (sequence, tile of 32 consecutive query rows, KV head, chunk of up to four of its query heads);
-// wave w takes query head w of the chunk.  The keys and values from the first row's window start
-// to the last row walk through LDS in tiles of 32, staged once for all waves: keys row-major for
-// the first product, values transposed for the second.
+// kv_attention_tile_kernel<S, DB, VB>: runs of rows (prompts, portions), on 32x32x16 MFMAs.  One
+// workgroup per (sequence, tile of query rows, KV head, chunk of its query heads).  Its four waves
+// are (query head of the chunk) x (block of 32 consecutive rows): 4 x 1 for groups of three heads
+// and more, 2 x 2 for two, 1 x 4 for one, so a tile is 32, 64 or 128 rows.  Keys and values from
+// the first row's window start to the last row walk through LDS in tiles of 64, row-major, staged
+// once for all waves and loaded one tile ahead; the rows' places in the paged caches are looked up
+// once per tile by 64 threads, two tiles ahead.
+//   S^T = K q^T   A = K    lane: key c of a 32-key block, dims 16 ks + 8 hf .. + 7   (LDS, 16 bytes)
+//                 B = q^T  lane: query c, the same dims (registers, loaded once)
+//                 C        lane: query c, keys (i & 3) + 8 (i >> 2) + 4 hf, i = 0 .. 15
+//   O^T = V^T P^T B = P^T  lane: query c, registers 8 s .. 8 s + 7 of C = keys 16 s + 4 hf + {0..3, 8..11}
+//                 A = V^T  lane: value dim 32 n + c of the same eight keys (16-bit reads down a
+//                          column of the row-major tile; neighbouring lanes read neighbouring
+//                          elements)
+// The k index of the second product is a free relabelling of the keys, so the weights go from the
+// first product's result to the second's operand without leaving the lane.  Scores, running
+// max / sum (base 2) and the accumulators are fp32; a weight enters the second product rounded to
+// the model dtype.
+template <class S>
+struct Mfma16;
+template <>
+struct Mfma16<BF16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                   c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma16<F16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c,
+                                                  0, 0, 0);
+  }
+};
+
+constexpr int kKeys = 64;     // keys per staged tile
+
 template <class S, int DB, int VB>
 __global__ __launch_bounds__(256) void kv_attention_tile_kernel(
     typename S::T* __restrict__ out, int64_t out_stride, const typename S::T* __restrict__ q,
@@ -316,35 +348,43 @@ __global__ __launch_bounds__(256) void kv_attention_tile_kernel(
     const typename S::T* __restrict__ key_cache, const typename S::T* __restrict__ value_cache,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ query_start_loc,
     const int* __restrict__ context_lens, const float* __restrict__ out_inv_freq, int interleaved,
-    int heads, int kv_heads, int block_size, int num_blocks, int window, float scale) {
+    int heads, int kv_heads, int block_size, int num_blocks, int window, float scale, int head_waves) {
   using T = typename S::T;
-  using M = Mfma8<S>;
+  using M = Mfma16<S>;
   constexpr int D = 32 * DB, VD = 32 * VB;
-  constexpr int KROW = D + 4, TROW = kTile + 4;      // elements; both keep 8-byte alignment
-  __shared__ __align__(16) T k_lds[kTile * KROW];    // [key][dim]
-  __shared__ __align__(16) T vt_lds[VD * TROW];      // [value dim][key]
+  constexpr int KROW = D + 8, VROW = VD + 8;          // elements; rows stay 16-byte aligned
+  __shared__ __align__(16) T k_lds[kKeys * KROW];
+  __shared__ __align__(16) T v_lds[kKeys * VROW];
+  __shared__ long long rows_lds[2][kKeys];            // token row of each key of a tile, -1: none
   const int b = blockIdx.z;
-  const int t0 = query_start_loc[b] + kTile * blockIdx.x;
-  const int nq = min(kTile, query_start_loc[b + 1] - t0);
-  if (nq <= 0) return;
+  const int row_blocks = 4 / head_waves;              // blocks of 32 query rows per workgroup
+  const int tile_rows = kTile * row_blocks;
+  const int t_first = query_start_loc[b] + tile_rows * blockIdx.x;
+  const int n_tile = min(tile_rows, query_start_loc[b + 1] - t_first);
+  if (n_tile <= 0) return;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int hf = lane >> 5, c = lane & 31;
   const int group = heads / kv_heads;
-  const int chunks = (group + 3) / 4;
+  const int chunks = (group + head_waves - 1) / head_waves;
   const int g = blockIdx.y / chunks;
-  const int h = g * group + (blockIdx.y % chunks) * 4 + w;
-  const bool active = h < g * group + group;
-  const int p0 = context_lens[b] + kTile * blockIdx.x, p_last = p0 + nq - 1;
-  const int j_lo = window > 0 ? max(0, p0 - window + 1) : 0;
-  const int* table = block_tables + (int64_t)b * max_blocks;
+  const int h = g * group + (blockIdx.y % chunks) * head_waves + w % head_waves;
+  const int rb = w / head_waves;                      // this wave's block of rows
+  const int t0 = t_first + kTile * rb;
+  const int nq = min(kTile, n_tile - kTile * rb);     // <= 0: no rows for this wave
+  const bool active = h < g * group + group && nq > 0;
+  const int p_first = context_lens[b] + tile_rows * blockIdx.x, p_last = p_first + n_tile - 1;
+  const int p0 = p_first + kTile * rb;                // this wave's first position
   const int pq = p0 + c;
+  const int j_lo = window > 0 ? max(0, p_first - window + 1) : 0;
+  const int* table = block_tables + (int64_t)b * max_blocks;
+  const float scale2 = scale * 1.4426950408889634f;   // scores in base 2
 
-  u32x2 qf[D / 8];
+  u32x4 qf[D / 16];
 #pragma unroll
-  for (int ks = 0; ks < D / 8; ++ks) {
-    u32x2 v = {0u, 0u};
+  for (int ks = 0; ks < D / 16; ++ks) {
+    u32x4 v = {0u, 0u, 0u, 0u};
     if (active && c < nq)
-      v = *reinterpret_cast<const u32x2*>(q + (int64_t)(t0 + c) * q_stride + (int64_t)h * D + 8 * ks + 4 * hf);
+      v = *reinterpret_cast<const u32x4*>(q + (int64_t)(t0 + c) * q_stride + (int64_t)h * D + 16 * ks + 8 * hf);
     qf[ks] = v;
   }
   f32x16 o[VB];
@@ -354,105 +394,130 @@ __global__ __launch_bounds__(256) void kv_attention_tile_kernel(
     for (int i = 0; i < 16; ++i) o[n][i] = 0.f;
   float m = -INFINITY, l = 0.f;
 
-  // staging: DB + VB pieces of 8 bytes per thread and tile, loaded one tile ahead
-  u32x2 xk[DB], xv[VB];
-  auto fetch = [&](int j0) {
-    auto token = [&](int j) {
+  auto look_up = [&](int j0, int buf) {               // threads 0 .. 63
+    const int j = j0 + tid;
+    long long row = -1;
+    if (j <= p_last) {
       int blk = table[j / block_size];
       blk = (unsigned)blk < (unsigned)num_blocks ? blk : 0;
-      return ((long long)blk * block_size + j % block_size) * kv_heads + g;
-    };
+      row = ((long long)blk * block_size + j % block_size) * kv_heads + g;
+    }
+    rows_lds[buf][tid] = row;
+  };
+  // staging: DB + VB pieces of 16 bytes per thread and tile
+  u32x4 xk[DB], xv[VB];
+  auto fetch = [&](int buf) {
 #pragma unroll
     for (int u = 0; u < DB; ++u) {
       const int i = tid + 256 * u;
-      const int r = i / (D / 4), v = i % (D / 4);
-      const int j = j0 + r;
-      const long long off = j <= p_last ? token(j) * D + 4 * v : 0;
-      const u32x2 got = *reinterpret_cast<const u32x2*>(key_cache + off);
-      xk[u] = j <= p_last ? got : u32x2{0u, 0u};
+      const int r = i / (D / 8), v = i % (D / 8);
+      const long long row = rows_lds[buf][r];
+      const u32x4 got = *reinterpret_cast<const u32x4*>(key_cache + (row >= 0 ? row * D + 8 * v : 0));
+      xk[u] = row >= 0 ? got : u32x4{0u, 0u, 0u, 0u};
     }
 #pragma unroll
     for (int u = 0; u < VB; ++u) {
       const int i = tid + 256 * u;
-      const int r = i / (VD / 4), v = i % (VD / 4);
-      const int j = j0 + r;
-      const long long off = j <= p_last ? token(j) * VD + 4 * v : 0;
-      const u32x2 got = *reinterpret_cast<const u32x2*>(value_cache + off);
-      xv[u] = j <= p_last ? got : u32x2{0u, 0u};
+      const int r = i / (VD / 8), v = i % (VD / 8);
+      const long long row = rows_lds[buf][r];
+      const u32x4 got = *reinterpret_cast<const u32x4*>(value_cache + (row >= 0 ? row * VD + 8 * v : 0));
+      xv[u] = row >= 0 ? got : u32x4{0u, 0u, 0u, 0u};
     }
   };
-  fetch(j_lo);
-  for (int j0 = j_lo; j0 <= p_last; j0 += kTile) {
-    __syncthreads();
+  if (tid < kKeys) {
+    look_up(j_lo, 0);
+    look_up(j_lo + kKeys, 1);
+  }
+  __syncthreads();
+  fetch(0);
+  int it = 0;
+  for (int j0 = j_lo; j0 <= p_last; j0 += kKeys, ++it) {
+    __syncthreads();          // the tiles of the step before are read; the next look-up is there
 #pragma unroll
     for (int u = 0; u < DB; ++u) {
       const int i = tid + 256 * u;
-      const int r = i / (D / 4), v = i % (D / 4);
-      *reinterpret_cast<u32x2*>(k_lds + r * KROW + 4 * v) = xk[u];
+      const int r = i / (D / 8), v = i % (D / 8);
+      *reinterpret_cast<u32x4*>(k_lds + r * KROW + 8 * v) = xk[u];
     }
 #pragma unroll
     for (int u = 0; u < VB; ++u) {
       const int i = tid + 256 * u;
-      const int r = i / (VD / 4), v = i % (VD / 4);
-      uint16_t* col = reinterpret_cast<uint16_t*>(vt_lds) + (4 * v) * TROW + r;
-      col[0] = (uint16_t)(xv[u][0] & 0xffffu);
-      col[TROW] = (uint16_t)(xv[u][0] >> 16);
-      col[2 * TROW] = (uint16_t)(xv[u][1] & 0xffffu);
-      col[3 * TROW] = (uint16_t)(xv[u][1] >> 16);
+      const int r = i / (VD / 8), v = i % (VD / 8);
+      *reinterpret_cast<u32x4*>(v_lds + r * VROW + 8 * v) = xv[u];
     }
-    if (j0 + kTile <= p_last) fetch(j0 + kTile);
+    if (j0 + kKeys <= p_last) fetch((it + 1) & 1);
     __syncthreads();
-    if (!active) continue;
-    f32x16 st;
+    if (tid < kKeys && j0 + 2 * kKeys <= p_last) look_up(j0 + 2 * kKeys, it & 1);
+    // keys past this wave's last row, or before its first row's window, are none of its business
+    if (!active || j0 > p0 + nq - 1 || (window > 0 && j0 + kKeys - 1 < p0 - window + 1)) continue;
+    f32x16 st[2];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) st[i] = 0.f;
+    for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-    for (int ks = 0; ks < D / 8; ++ks) {
-      const u32x2 a = *reinterpret_cast<const u32x2*>(k_lds + c * KROW + 8 * ks + 4 * hf);
-      st = M::run(a, qf[ks], st);
+      for (int i = 0; i < 16; ++i) st[kb][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        const u32x4 a = *reinterpret_cast<const u32x4*>(k_lds + (32 * kb + c) * KROW + 16 * ks + 8 * hf);
+        st[kb] = M::run(a, qf[ks], st[kb]);
+      }
     }
+    // every key of the tile visible to every row of the wave: no masks
+    const bool full = j0 + kKeys - 1 <= p0 && nq == kTile && (window <= 0 || p0 + kTile - 1 - j0 < window);
     float mt = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int key = j0 + (i & 3) + 8 * (i >> 2) + 4 * hf;
-      const int dist = pq - key;
-      const bool ok = c < nq && dist >= 0 && (window <= 0 || dist < window);
-      st[i] = ok ? st[i] * scale : -INFINITY;
-      mt = fmaxf(mt, st[i]);
-    }
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float v = st[kb][i] * scale2;
+        if (!full) {
+          const int dist = pq - (j0 + 32 * kb + (i & 3) + 8 * (i >> 2) + 4 * hf);
+          const bool ok = c < nq && dist >= 0 && (window <= 0 || dist < window);
+          v = ok ? v : -INFINITY;
+        }
+        st[kb][i] = v;
+        mt = fmaxf(mt, v);
+      }
     mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
     const float m_new = fmaxf(m, mt);
-    const float corr = m_new == -INFINITY ? 1.f : expf(m - m_new);
+    const bool none = m_new == -INFINITY;
+    const float corr = none ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
     float psum = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      st[i] = m_new == -INFINITY ? 0.f : expf(st[i] - m_new);
-      psum += st[i];
-    }
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float pv = none ? 0.f : __builtin_amdgcn_exp2f(st[kb][i] - m_new);
+        st[kb][i] = pv;
+        psum += pv;
+      }
     l = l * corr + psum;          // this lane's keys; the partner's half is added at the end
     m = m_new;
+    if (__any(corr != 1.f)) {      // the running max of some row moved
 #pragma unroll
-    for (int n = 0; n < VB; ++n)
+      for (int n = 0; n < VB; ++n)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) o[n][i] *= corr;
-#pragma unroll
-    for (int s8 = 0; s8 < 4; ++s8) {
-      uint32_t hb[4], lb[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float pv = st[4 * s8 + e];
-        hb[e] = bits16<S>(pv);
-        lb[e] = bits16<S>(pv - from_bits16<S>(hb[e]));
-      }
-      const u32x2 hi = {hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16)};
-      const u32x2 lo = {lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16)};
-#pragma unroll
-      for (int n = 0; n < VB; ++n) {
-        const u32x2 a = *reinterpret_cast<const u32x2*>(vt_lds + (32 * n + c) * TROW + 8 * s8 + 4 * hf);
-        o[n] = M::run(a, hi, o[n]);
-        o[n] = M::run(a, lo, o[n]);
-      }
+        for (int i = 0; i < 16; ++i) o[n][i] *= corr;
     }
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        u32x4 pb;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          pb[e] = bits16<S>(st[kb][8 * s2 + 2 * e]) | (bits16<S>(st[kb][8 * s2 + 2 * e + 1]) << 16);
+        const uint16_t* col0 = reinterpret_cast<const uint16_t*>(v_lds) + (32 * kb + 16 * s2 + 4 * hf) * VROW + c;
+#pragma unroll
+        for (int n = 0; n < VB; ++n) {
+          const uint16_t* col = col0 + 32 * n;
+          u32x4 a;
+          a[0] = (uint32_t)col[0] | ((uint32_t)col[VROW] << 16);
+          a[1] = (uint32_t)col[2 * VROW] | ((uint32_t)col[3 * VROW] << 16);
+          a[2] = (uint32_t)col[8 * VROW] | ((uint32_t)col[9 * VROW] << 16);
+          a[3] = (uint32_t)col[10 * VROW] | ((uint32_t)col[11 * VROW] << 16);
+          o[n] = M::run(a, pb, o[n]);
+        }
+      }
   }
   if (!active) return;
   l += __shfl_xor(l, 32, 64);
@@ -704,11 +769,11 @@ int launch_tiles_one(dim3 grid, hipStream_t stream, typename S::T* out, int64_t 
                      const typename S::T* value_cache, const int* block_tables, int max_blocks,
                      const int* qsl, const int* ctx, const float* out_inv_freq, int interleaved,
                      int heads, int kv_heads, int block_size, int num_blocks, int window,
-                     float scale) {
+                     float scale, int head_waves) {
   kv_attention_tile_kernel<S, DB, VB><<<grid, 256, 0, stream>>>(
       out, out_stride, q, q_stride, gate, gate_stride, key_cache, value_cache, block_tables,
       max_blocks, qsl, ctx, out_inv_freq, interleaved, heads, kv_heads, block_size, num_blocks,
-      window, scale);
+      window, scale, head_waves);
   VLA_SEQ_HIP_CHECK(hipGetLastError());
   return VLA_OK;
 }
@@ -855,17 +920,24 @@ extern "C" int vla_seq_kv_attention_tiles(
   if (((uintptr_t)q % 8) || ((q_stride * 2) % 8) || ((uintptr_t)key_cache % 8) ||
       ((uintptr_t)value_cache % 8))
     return VLA_ERR_ARG;
+  // 16-byte fragment loads: query rows and cache rows must allow them
+  if (((uintptr_t)q % 16) || ((q_stride * 2) % 16) || ((uintptr_t)key_cache % 16) ||
+      ((uintptr_t)value_cache % 16))
+    return VLA_ERR_ARG;
   const int group = heads / kv_heads;
-  const dim3 grid((max_query_len + kTile - 1) / kTile, kv_heads * ((group + 3) / 4), num_seqs);
+  const int head_waves = group >= 3 ? 4 : group;      // waves of a workgroup that are heads
+  const int tile_rows = kTile * (4 / head_waves);
+  const dim3 grid((max_query_len + tile_rows - 1) / tile_rows,
+                  kv_heads * ((group + head_waves - 1) / head_waves), num_seqs);
   if (dtype == VLA_BF16)
     return launch_tiles<BF16>(dim / 32, vdim / 32, grid, (hipStream_t)stream, (__bf16*)out, out_stride,
                               (const __bf16*)q, q_stride, (const __bf16*)gate, gate_stride,
                               (const __bf16*)key_cache, (const __bf16*)value_cache, block_tables,
                               max_blocks, query_start_loc, context_lens, out_inv_freq, interleaved,
-                              heads, kv_heads, block_size, num_blocks, window, scale);
+                              heads, kv_heads, block_size, num_blocks, window, scale, head_waves);
   return launch_tiles<F16>(dim / 32, vdim / 32, grid, (hipStream_t)stream, (_Float16*)out, out_stride,
                            (const _Float16*)q, q_stride, (const _Float16*)gate, gate_stride,
                            (const _Float16*)key_cache, (const _Float16*)value_cache, block_tables,
                            max_blocks, query_start_loc, context_lens, out_inv_freq, interleaved, heads,
-                           kv_heads, block_size, num_blocks, window, scale);
+                           kv_heads, block_size, num_blocks, window, scale, head_waves);
 }
