@@ -315,9 +315,8 @@ __device__ __forceinline__ void turn_back(f32x16 (&o)[VB], int hf, float p,
 //                 B = q^T  lane: query c, the same dims (registers, loaded once)
 //                 C        lane: query c, keys (i & 3) + 8 (i >> 2) + 4 hf, i = 0 .. 15
 //   O^T = V^T P^T B = P^T  lane: query c, registers 8 s .. 8 s + 7 of C = keys 16 s + 4 hf + {0..3, 8..11}
-//                 A = V^T  lane: value dim 32 n + c of the same eight keys (16-bit reads down a
-//                          column of the row-major tile; neighbouring lanes read neighbouring
-//                          elements)
+//                 A = V^T  lane: value dim 32 n + c of the same eight keys (two transposing reads
+//                          of the row-major tile)
 // The k index of the second product is a free relabelling of the keys, so the weights go from the
 // first product's result to the second's operand without leaving the lane.  Scores, running
 // max / sum (base 2) and the accumulators are fp32; a weight enters the second product rounded to
@@ -340,9 +339,25 @@ struct Mfma16<F16> {
 };
 
 constexpr int kKeys = 64;     // keys per staged tile
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef s16x4 __attribute__((address_space(3))) * lds_s16x4;
+
+// two fp32 -> one word of two model-dtype values (round to nearest even), as one packed convert
+template <class S>
+__device__ __forceinline__ uint32_t pack2(float a, float b);
+template <>
+__device__ __forceinline__ uint32_t pack2<F16>(float a, float b) {
+  const f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<BF16>(float a, float b) {
+  const f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
 
 template <class S, int DB, int VB>
-__global__ __launch_bounds__(256) void kv_attention_tile_kernel(
+__global__ __launch_bounds__(256, 2) void kv_attention_tile_kernel(
     typename S::T* __restrict__ out, int64_t out_stride, const typename S::T* __restrict__ q,
     int64_t q_stride, const typename S::T* __restrict__ gate, int64_t gate_stride,
     const typename S::T* __restrict__ key_cache, const typename S::T* __restrict__ value_cache,
@@ -352,9 +367,11 @@ __global__ __launch_bounds__(256) void kv_attention_tile_kernel(
   using T = typename S::T;
   using M = Mfma16<S>;
   constexpr int D = 32 * DB, VD = 32 * VB;
-  constexpr int KROW = D + 8, VROW = VD + 8;          // elements; rows stay 16-byte aligned
-  __shared__ __align__(16) T k_lds[kKeys * KROW];
-  __shared__ __align__(16) T v_lds[kKeys * VROW];
+  // elements; rows stay 16-byte aligned, and four value rows a transposing read takes fall into
+  // different banks
+  constexpr int KROW = D + 8, VROW = VD + 16;
+  __shared__ __align__(16) T k_lds2[2][kKeys * KROW];  // two tiles: one is read while the next lands
+  __shared__ __align__(16) T v_lds2[2][kKeys * VROW];
   __shared__ long long rows_lds[2][kKeys];            // token row of each key of a tile, -1: none
   const int b = blockIdx.z;
   const int row_blocks = 4 / head_waves;              // blocks of 32 query rows per workgroup
@@ -394,15 +411,19 @@ __global__ __launch_bounds__(256) void kv_attention_tile_kernel(
     for (int i = 0; i < 16; ++i) o[n][i] = 0.f;
   float m = -INFINITY, l = 0.f;
 
-  auto look_up = [&](int j0, int buf) {               // threads 0 .. 63
+  // threads 0 .. 63 look the rows of a tile up: the block id is read one step before it is used
+  auto load_block = [&](int j0) {
     const int j = j0 + tid;
-    long long row = -1;
+    int blk = -1;
     if (j <= p_last) {
-      int blk = table[j / block_size];
+      blk = table[j / block_size];
       blk = (unsigned)blk < (unsigned)num_blocks ? blk : 0;
-      row = ((long long)blk * block_size + j % block_size) * kv_heads + g;
     }
-    rows_lds[buf][tid] = row;
+    return blk;
+  };
+  auto store_row = [&](int j0, int blk, int buf) {
+    const int j = j0 + tid;
+    rows_lds[buf][tid] = blk < 0 ? -1 : ((long long)blk * block_size + j % block_size) * kv_heads + g;
   };
   // staging: DB + VB pieces of 16 bytes per thread and tile
   u32x4 xk[DB], xv[VB];
@@ -424,100 +445,122 @@ __global__ __launch_bounds__(256) void kv_attention_tile_kernel(
       xv[u] = row >= 0 ? got : u32x4{0u, 0u, 0u, 0u};
     }
   };
-  if (tid < kKeys) {
-    look_up(j_lo, 0);
-    look_up(j_lo + kKeys, 1);
-  }
-  __syncthreads();
-  fetch(0);
-  int it = 0;
-  for (int j0 = j_lo; j0 <= p_last; j0 += kKeys, ++it) {
-    __syncthreads();          // the tiles of the step before are read; the next look-up is there
+  auto land = [&](int buf) {                           // the fetched tile into LDS
 #pragma unroll
     for (int u = 0; u < DB; ++u) {
       const int i = tid + 256 * u;
       const int r = i / (D / 8), v = i % (D / 8);
-      *reinterpret_cast<u32x4*>(k_lds + r * KROW + 8 * v) = xk[u];
+      *reinterpret_cast<u32x4*>(k_lds2[buf] + r * KROW + 8 * v) = xk[u];
     }
 #pragma unroll
     for (int u = 0; u < VB; ++u) {
       const int i = tid + 256 * u;
       const int r = i / (VD / 8), v = i % (VD / 8);
-      *reinterpret_cast<u32x4*>(v_lds + r * VROW + 8 * v) = xv[u];
+      *reinterpret_cast<u32x4*>(v_lds2[buf] + r * VROW + 8 * v) = xv[u];
     }
-    if (j0 + kKeys <= p_last) fetch((it + 1) & 1);
-    __syncthreads();
-    if (tid < kKeys && j0 + 2 * kKeys <= p_last) look_up(j0 + 2 * kKeys, it & 1);
+  };
+  // One barrier per tile.  At the top of step `it`: tile `it` is in LDS buffer it & 1, tile it + 1
+  // in the staging registers, the rows of tile it + 2 in rows_lds[it & 1], and threads 0 .. 63 hold
+  // the block ids of tile it + 3 (whose rows go to rows_lds[(it + 1) & 1] during the step).
+  int blk_next = -1;
+  if (tid < kKeys) {
+    store_row(j_lo, load_block(j_lo), 0);
+    store_row(j_lo + kKeys, load_block(j_lo + kKeys), 1);
+  }
+  __syncthreads();
+  fetch(0);
+  land(0);
+  fetch(1);
+  __syncthreads();                                     // rows_lds[0] is read: tile 2's rows may go there
+  if (tid < kKeys) {
+    store_row(j_lo + 2 * kKeys, load_block(j_lo + 2 * kKeys), 0);
+    blk_next = load_block(j_lo + 3 * kKeys);
+  }
+  __syncthreads();
+  int it = 0;
+  for (int j0 = j_lo; j0 <= p_last; j0 += kKeys, ++it) {
+    const T* k_lds = k_lds2[it & 1];
+    const T* v_lds = v_lds2[it & 1];
     // keys past this wave's last row, or before its first row's window, are none of its business
-    if (!active || j0 > p0 + nq - 1 || (window > 0 && j0 + kKeys - 1 < p0 - window + 1)) continue;
-    f32x16 st[2];
+    if (active && j0 <= p0 + nq - 1 && !(window > 0 && j0 + kKeys - 1 < p0 - window + 1)) {
+      f32x16 st[2];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+      for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) st[kb][i] = 0.f;
+        for (int i = 0; i < 16; ++i) st[kb][i] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks) {
-        const u32x4 a = *reinterpret_cast<const u32x4*>(k_lds + (32 * kb + c) * KROW + 16 * ks + 8 * hf);
-        st[kb] = M::run(a, qf[ks], st[kb]);
-      }
-    }
-    // every key of the tile visible to every row of the wave: no masks
-    const bool full = j0 + kKeys - 1 <= p0 && nq == kTile && (window <= 0 || p0 + kTile - 1 - j0 < window);
-    float mt = -INFINITY;
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float v = st[kb][i] * scale2;
-        if (!full) {
-          const int dist = pq - (j0 + 32 * kb + (i & 3) + 8 * (i >> 2) + 4 * hf);
-          const bool ok = c < nq && dist >= 0 && (window <= 0 || dist < window);
-          v = ok ? v : -INFINITY;
-        }
-        st[kb][i] = v;
-        mt = fmaxf(mt, v);
-      }
-    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-    const float m_new = fmaxf(m, mt);
-    const bool none = m_new == -INFINITY;
-    const float corr = none ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
-    float psum = 0.f;
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float pv = none ? 0.f : __builtin_amdgcn_exp2f(st[kb][i] - m_new);
-        st[kb][i] = pv;
-        psum += pv;
-      }
-    l = l * corr + psum;          // this lane's keys; the partner's half is added at the end
-    m = m_new;
-    if (__any(corr != 1.f)) {      // the running max of some row moved
-#pragma unroll
-      for (int n = 0; n < VB; ++n)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[n][i] *= corr;
-    }
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-        u32x4 pb;
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          pb[e] = bits16<S>(st[kb][8 * s2 + 2 * e]) | (bits16<S>(st[kb][8 * s2 + 2 * e + 1]) << 16);
-        const uint16_t* col0 = reinterpret_cast<const uint16_t*>(v_lds) + (32 * kb + 16 * s2 + 4 * hf) * VROW + c;
-#pragma unroll
-        for (int n = 0; n < VB; ++n) {
-          const uint16_t* col = col0 + 32 * n;
-          u32x4 a;
-          a[0] = (uint32_t)col[0] | ((uint32_t)col[VROW] << 16);
-          a[1] = (uint32_t)col[2 * VROW] | ((uint32_t)col[3 * VROW] << 16);
-          a[2] = (uint32_t)col[8 * VROW] | ((uint32_t)col[9 * VROW] << 16);
-          a[3] = (uint32_t)col[10 * VROW] | ((uint32_t)col[11 * VROW] << 16);
-          o[n] = M::run(a, pb, o[n]);
+        for (int ks = 0; ks < D / 16; ++ks) {
+          const u32x4 a = *reinterpret_cast<const u32x4*>(k_lds + (32 * kb + c) * KROW + 16 * ks + 8 * hf);
+          st[kb] = M::run(a, qf[ks], st[kb]);
         }
       }
+      // every key of the tile visible to every row of the wave: no masks
+      const bool full = j0 + kKeys - 1 <= p0 && nq == kTile && (window <= 0 || p0 + kTile - 1 - j0 < window);
+      float mt = -INFINITY;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          float v = st[kb][i] * scale2;
+          if (!full) {
+            const int dist = pq - (j0 + 32 * kb + (i & 3) + 8 * (i >> 2) + 4 * hf);
+            const bool ok = c < nq && dist >= 0 && (window <= 0 || dist < window);
+            v = ok ? v : -INFINITY;
+          }
+          st[kb][i] = v;
+          mt = fmaxf(mt, v);
+        }
+      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      const float m_new = fmaxf(m, mt);
+      const bool none = m_new == -INFINITY;
+      const float corr = none ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+      float psum = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const float pv = none ? 0.f : __builtin_amdgcn_exp2f(st[kb][i] - m_new);
+          st[kb][i] = pv;
+          psum += pv;
+        }
+      l = l * corr + psum;          // this lane's keys; the partner's half is added at the end
+      m = m_new;
+      if (__any(corr != 1.f)) {     // the running max of some row moved
+#pragma unroll
+        for (int n = 0; n < VB; ++n)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[n][i] *= corr;
+      }
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          u32x4 pb;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) pb[e] = pack2<S>(st[kb][8 * s2 + 2 * e], st[kb][8 * s2 + 2 * e + 1]);
+          // transposing read of the row-major tile: a group of 16 lanes reads 4 keys x 16 dims, 8
+          // bytes per lane (key i16 >> 2, dims 4 (i16 & 3) .. + 3), and every lane receives the four
+          // keys of dim i16 of the group
+          const int i16 = c & 15;
+          const T* src = v_lds + (32 * kb + 16 * s2 + 4 * hf + (i16 >> 2)) * VROW + 16 * (c >> 4) + 4 * (i16 & 3);
+#pragma unroll
+          for (int n = 0; n < VB; ++n) {
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)(src + 32 * n));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)(src + 32 * n + 8 * VROW));
+            const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
+            const u32x4 a = {lo2[0], lo2[1], hi2[0], hi2[1]};
+            o[n] = M::run(a, pb, o[n]);
+          }
+        }
+    }
+    if (j0 + kKeys <= p_last) land((it + 1) & 1);              // tile it + 1, fetched a step ago
+    if (j0 + 2 * kKeys <= p_last) fetch(it & 1);               // tile it + 2 on its way
+    if (tid < kKeys && j0 + 3 * kKeys <= p_last) {
+      // rows of tile it + 3 into the buffer the step before read tile it + 1's from
+      store_row(j0 + 3 * kKeys, blk_next, (it + 1) & 1);
+      blk_next = load_block(j0 + 4 * kKeys);
+    }
+    __syncthreads();
   }
   if (!active) return;
   l += __shfl_xor(l, 32, 64);
