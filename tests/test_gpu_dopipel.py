@@ -368,6 +368,11 @@ def test_activations(act):
     assert float((got - f(g) * u).abs().max()) <= 1e-5
     got = GatedActivation(act, gated=False)(z.to(DEV)).cpu()
     assert float((got - f(z.to(F))).abs().max()) <= 1e-5
+    # 16-bit rows of a multiple of eight values take the vector form
+    zb = rnd((5, 2 * 72), 1, 2.0).to(torch.bfloat16)
+    got = GatedActivation(act)(zb.to(DEV)).float().cpu()
+    want = f(zb[:, :72].to(F)) * zb[:, 72:].to(F)
+    assert float((got - want).abs().max()) <= 0.02 * float(want.abs().max())
 
 
 MOE_SHAPES = [
@@ -378,6 +383,8 @@ MOE_SHAPES = [
     (96, 12, 2, 2, 64, 96),
     (72, 5, 3, 4, 130, 0),
     (50, 4, 1, 2, 9, 7),       # sizes the matrix-core product does not take: the plain one runs
+    (72, 2, 0, 1, 40, 0),      # multiples of 8 but not of 16: the narrower matrix-core product
+    (64, 2, 0, 2, 48, 16),     # two experts, both chosen: long runs of tiles of one expert
 ]
 
 
@@ -391,7 +398,7 @@ def test_routed_experts(shape, dtype):
     t = R.sub(R.make_weights(cfg, seed=3), "l0.mlp.")
     layer = RoutedExperts(W, E, I, top, ff, sff, dtype=dtype, device=DEV)
     layer.set_weights(t)
-    for T in (1, 2, 33, 150):
+    for T in (1, 2, 33, 150, 300):
         h = rnd((T, W), T).to(dtype)
         tt = {k: v.to(F) for k, v in t.items()}
         want = R.moe_ff(h.to(F), tt, mlp)

@@ -22,8 +22,14 @@ __global__ __launch_bounds__(kThreads) void residual_norms_kernel(
     const float* __restrict__ pre_w, float eps, int width) {
   __shared__ float red[16];
   const int64_t base = (int64_t)blockIdx.x * width;
-  float keep[kKeep];
+  float keep[kKeep], keepx[kKeep];
   float inv_y = 0.f;
+  // the stream's row is asked for before the first reduction, so its latency hides behind it
+#pragma unroll
+  for (int i = 0; i < kKeep; ++i) {
+    const int c = threadIdx.x + i * kThreads;
+    keepx[i] = c < width ? x[base + c] : 0.f;
+  }
   if (y != nullptr) {
     const typename SY::T* yr = y + (int64_t)blockIdx.x * y_stride;
     float ss = 0.f;
@@ -44,8 +50,8 @@ __global__ __launch_bounds__(kThreads) void residual_norms_kernel(
   }
   const bool writes = y != nullptr || add_row != nullptr;
   float ss = 0.f;
-  auto update = [&](int c, float yv) {
-    float v = x[base + c];
+  auto update = [&](int c, float xv, float yv) {
+    float v = xv;
     if (y != nullptr) {
       float u = yv * inv_y * post_w[c];
       if (layer_scale != nullptr) u *= layer_scale[c];
@@ -59,12 +65,12 @@ __global__ __launch_bounds__(kThreads) void residual_norms_kernel(
 #pragma unroll
   for (int i = 0; i < kKeep; ++i) {
     const int c = threadIdx.x + i * kThreads;
-    if (c < width) keep[i] = update(c, y != nullptr ? keep[i] : 0.f);
+    if (c < width) keep[i] = update(c, keepx[i], y != nullptr ? keep[i] : 0.f);
   }
   for (int c = threadIdx.x + kKeep * kThreads; c < width; c += kThreads)
-    update(c, y != nullptr ? SY::to_f32(y[(int64_t)blockIdx.x * y_stride + c]) +
-                                 (y_bias != nullptr ? y_bias[c] : 0.f)
-                           : 0.f);
+    update(c, x[base + c], y != nullptr ? SY::to_f32(y[(int64_t)blockIdx.x * y_stride + c]) +
+                                              (y_bias != nullptr ? y_bias[c] : 0.f)
+                                        : 0.f);
   if (out == nullptr) return;
   ss = block_sum(ss, red);
   const float inv = 1.f / sqrtf(ss / (float)width + eps);
@@ -167,6 +173,32 @@ __global__ __launch_bounds__(kThreads) void gated_act_kernel(
   out[t * out_stride + c] = S::from_f32(v);
 }
 
+// 16-bit rows whose length is a multiple of eight and whose ends are 16-byte aligned: eight values
+// per access, a workgroup per row
+template <class S>
+__global__ __launch_bounds__(kThreads) void gated_act_vec_kernel(
+    typename S::T* __restrict__ out, int64_t out_stride, const typename S::T* __restrict__ gate,
+    int64_t gate_stride, const typename S::T* __restrict__ up, int64_t up_stride, int features,
+    int act) {
+  const int64_t t = blockIdx.x;
+  for (int c = 8 * threadIdx.x; c < features; c += 8 * kThreads) {
+    const u32x4 g = *reinterpret_cast<const u32x4*>(gate + t * gate_stride + c);
+    u32x4 u = {0u, 0u, 0u, 0u};
+    if (up != nullptr) u = *reinterpret_cast<const u32x4*>(up + t * up_stride + c);
+    u32x4 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float a = activate(lo16<S>(g[e]), act), b = activate(hi16<S>(g[e]), act);
+      if (up != nullptr) {
+        a *= lo16<S>(u[e]);
+        b *= hi16<S>(u[e]);
+      }
+      r[e] = pack16<S>(a, b);
+    }
+    *reinterpret_cast<u32x4*>(out + t * out_stride + c) = r;
+  }
+}
+
 template <class F>
 int with_two_dtypes(int a, int b, F&& f) {
   return with_dtype(a, [&](auto sa) { return with_dtype(b, [&](auto sb) { return f(sa, sb); }); });
@@ -249,6 +281,18 @@ extern "C" int vla_seq_gated_act(void* out, int64_t out_stride, const void* gate
     return VLA_ERR_ARG;
   return with_dtype(dtype, [&](auto s) {
     using S = decltype(s);
+    if constexpr (sizeof(typename S::T) == 2) {
+      const bool ok = features % 8 == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)gate % 16) == 0 &&
+                      (!up || ((uintptr_t)up % 16) == 0) && out_stride % 8 == 0 &&
+                      gate_stride % 8 == 0 && (!up || up_stride % 8 == 0);
+      if (ok) {
+        gated_act_vec_kernel<S><<<num_tokens, kThreads, 0, (hipStream_t)stream>>>(
+            (typename S::T*)out, out_stride, (const typename S::T*)gate, gate_stride,
+            (const typename S::T*)up, up_stride, features, act);
+        VLA_SEQ_HIP_CHECK(hipGetLastError());
+        return VLA_OK;
+      }
+    }
     gated_act_kernel<S><<<dim3(num_tokens, (features + kThreads - 1) / kThreads), kThreads, 0,
                           (hipStream_t)stream>>>((typename S::T*)out, out_stride,
                                                  (const typename S::T*)gate, gate_stride,

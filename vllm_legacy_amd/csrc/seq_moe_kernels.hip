@@ -216,6 +216,101 @@ __global__ __launch_bounds__(256) void grouped_linear_mfma_kernel(
   }
 }
 
+// The same product on 32x32x16 MFMAs (k_in a multiple of 16, 16-byte fragments) with up to kRunTiles
+// consecutive row tiles per workgroup: tiles of one expert share the weight fragment a wave has in
+// registers, so the weights are read once per run of tiles instead of once per tile.  A workgroup
+// walks its tiles in runs of equal expert.
+constexpr int kRunTiles = 4;
+
+template <class S>
+struct Mma16;
+template <>
+struct Mma16<BF16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                   c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma16<F16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c,
+                                                  0, 0, 0);
+  }
+};
+
+template <class S, class SO, int C>
+__device__ __forceinline__ void grouped_run(typename SO::T* __restrict__ out, int64_t out_stride,
+                                            const typename S::T* __restrict__ a, int64_t a_stride,
+                                            const int* __restrict__ row_token,
+                                            const typename S::T* __restrict__ wr, int first_tile, int n0,
+                                            int n_out, int k_in, int act, int hf, int c) {
+  using T = typename S::T;
+  const T* ar[C];
+  bool live[C];
+  f32x16 acc[C];
+#pragma unroll
+  for (int r = 0; r < C; ++r) {
+    const int row = (first_tile + r) * kTile + c;
+    const int src = row_token != nullptr ? row_token[row] : row;
+    live[r] = src >= 0;
+    ar[r] = a + (int64_t)(src < 0 ? 0 : src) * a_stride + 8 * hf;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[r][i] = 0.f;
+  }
+#pragma unroll 4
+  for (int k = 0; k < k_in; k += 16) {
+    const u32x4 wv = *reinterpret_cast<const u32x4*>(wr + k);
+#pragma unroll
+    for (int r = 0; r < C; ++r) {
+      u32x4 av = *reinterpret_cast<const u32x4*>(ar[r] + k);
+      if (!live[r]) av = u32x4{0u, 0u, 0u, 0u};
+      acc[r] = Mma16<S>::run(wv, av, acc[r]);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < C; ++r) {
+    const int row = (first_tile + r) * kTile + c;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int n = n0 + (i & 3) + 8 * (i >> 2) + 4 * hf;
+      if (n < n_out) out[(int64_t)row * out_stride + n] = SO::from_f32(act_apply(acc[r][i], act));
+    }
+  }
+}
+
+template <class S, class SO>
+__global__ __launch_bounds__(256) void grouped_linear_mfma16_kernel(
+    typename SO::T* __restrict__ out, int64_t out_stride, const typename S::T* __restrict__ a,
+    int64_t a_stride, const int* __restrict__ row_token, const typename S::T* __restrict__ weight,
+    const int* __restrict__ tile_expert, int max_tiles, int n_out, int k_in, int act,
+    int tiles_per_group) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int hf = lane >> 5, c = lane & 31;
+  const int n0 = (blockIdx.y * (blockDim.x >> 6) + w) * 32;
+  if (n0 >= n_out) return;
+  const int first = blockIdx.x * tiles_per_group;
+  const int last = min(first + tiles_per_group, max_tiles);
+  int i = first;
+  while (i < last) {
+    const int e = tile_expert[i];
+    if (e < 0) {
+      ++i;
+      continue;
+    }
+    int j = i + 1;
+    while (j < last && tile_expert[j] == e) ++j;
+    const typename S::T* wr = weight + ((int64_t)e * n_out + min(n0 + c, n_out - 1)) * k_in + 8 * hf;
+    switch (j - i) {
+      case 1: grouped_run<S, SO, 1>(out, out_stride, a, a_stride, row_token, wr, i, n0, n_out, k_in, act, hf, c); break;
+      case 2: grouped_run<S, SO, 2>(out, out_stride, a, a_stride, row_token, wr, i, n0, n_out, k_in, act, hf, c); break;
+      case 3: grouped_run<S, SO, 3>(out, out_stride, a, a_stride, row_token, wr, i, n0, n_out, k_in, act, hf, c); break;
+      default: grouped_run<S, SO, 4>(out, out_stride, a, a_stride, row_token, wr, i, n0, n_out, k_in, act, hf, c); break;
+    }
+    i = j;
+  }
+}
+
 // Any dtype and size, fp32 arithmetic: wave w of a workgroup takes eight rows of the tile, lane =
 // output column.
 template <class S, class SO>
@@ -333,6 +428,19 @@ extern "C" int vla_seq_grouped_linear(void* out, int64_t out_stride, int out_dty
     using T = typename S::T;
     hipStream_t st = (hipStream_t)stream;
     if constexpr (sizeof(T) == 2) {
+      if (k_in % 16 == 0 && ((uintptr_t)a % 16) == 0 && (a_stride % 8) == 0 && ((uintptr_t)weight % 16) == 0) {
+        // few tiles (decode steps): the launch is bound by reading each expert's weights once, so
+        // every (tile, 32 columns) is a one-wave workgroup of its own; many tiles: four waves
+        // and runs of tiles that share the weight fragments
+        const bool few = (int64_t)max_tiles * ((n_out + 127) / 128) <= 1024;
+        const int waves = few ? 1 : 4, per = few ? 1 : kRunTiles;
+        grouped_linear_mfma16_kernel<S, SO>
+            <<<dim3((max_tiles + per - 1) / per, (n_out + 32 * waves - 1) / (32 * waves)), 64 * waves, 0, st>>>(
+                (typename SO::T*)out, out_stride, (const T*)a, a_stride, row_token, (const T*)weight,
+                tile_expert, max_tiles, n_out, k_in, act, per);
+        VLA_SEQ_HIP_CHECK(hipGetLastError());
+        return VLA_OK;
+      }
       if (k_in % 8 == 0 && ((uintptr_t)a % 8) == 0 && (a_stride % 4) == 0 && ((uintptr_t)weight % 8) == 0) {
         grouped_linear_mfma_kernel<S, SO><<<dim3(max_tiles, (n_out + 127) / 128), 256, 0, st>>>(
             (typename SO::T*)out, out_stride, (const T*)a, a_stride, row_token, (const T*)weight,
