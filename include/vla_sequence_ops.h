@@ -151,7 +151,7 @@ int vla_seq_residual_norms(float* x, const void* y, int64_t y_stride, int y_dtyp
  *   out[t] = dtype(h[t] + sum_j weight[:, j] h[t - taps + 1 + j]),  zeros before a sequence's start,
  * h fp32 [T, width], weight fp32 [width, taps].  The last taps - 1 inputs of a sequence live in
  * state fp32 [num_slots, taps - 1, width] (oldest first): rows of earlier steps are read from
- * there, and the step leaves its own last inputs there.  taps <= 16. */
+ * there, and the step leaves its own last inputs there.  taps <= 32. */
 int vla_seq_causal_conv(void* out, const float* h, const float* weight, float* state,
                         const int* query_start_loc, const int* context_lens,
                         const int* state_slots, const int* token_seq, int num_tokens, int num_seqs,
@@ -233,12 +233,15 @@ int vla_seq_mingru_scan(void* out, int64_t out_stride, const void* zp, int64_t z
 
 /* Router of one token over `routed` experts (at most 512): z = router h in fp32 (router fp32
  * [routed, width]), s = softmax(z), the `top` largest s + correction (null: s) are chosen, weights
- * = their s / (sum + 1e-20).  experts int32 / weights fp32 [T, top].  shared_gate_weight fp32
- * [width] (null: none): shared_gate[t] = sigmoid(shared_gate_weight . h). */
-int vla_seq_moe_route(const void* h, int64_t h_stride, const float* router,
-                      const float* correction, const float* shared_gate_weight, int* experts,
-                      float* weights, float* shared_gate, int num_tokens, int width, int routed,
-                      int top, int dtype, void* stream);
+ * = their s / (sum + 1e-20).  experts int32 / weights fp32 [T, top].  shared_gate given:
+ * shared_gate[t] = sigmoid(shared_gate_weight . h), shared_gate_weight fp32 [width].  logits given
+ * (fp32 rows of routed (+ 1 with a shared gate, its logit last) values, stride logits_stride): the
+ * products are the caller's and h, router, shared_gate_weight are not read. */
+int vla_seq_moe_route(const void* h, int64_t h_stride, const float* router, const float* logits,
+                      int64_t logits_stride, const float* correction,
+                      const float* shared_gate_weight, int* experts, float* weights,
+                      float* shared_gate, int num_tokens, int width, int routed, int top, int dtype,
+                      void* stream);
 
 /* Groups the pairs (token, choice) whose expert is below num_experts by expert, every group padded
  * to whole tiles of vla_seq_moe_tile_rows() rows: pair_row int32 [T * top] (-1: the pair's expert

@@ -411,6 +411,11 @@ def test_routed_experts(shape, dtype):
         clear = (srt[:, :top] - srt[:, 1:top + 1]).min(-1).values > 1e-3 if top < E + I else torch.ones(T, dtype=torch.bool)
         assert torch.equal(torch.sort(ge.cpu()[clear].long(), -1).values, torch.sort(idx[clear], -1).values)
         got = layer(h.to(DEV)).cpu()
+        if T == 150:        # the same step with the router's logits from a matrix product
+            layer.ROUTE_PRODUCT_MIN_TOKENS = 100
+            other = layer(h.to(DEV)).cpu()
+            del layer.ROUTE_PRODUCT_MIN_TOKENS
+            assert float(((other - got).abs().max(-1).values / want.abs().max())[clear].max()) <= 1e-5
         bar = 2e-5 if dtype == torch.float32 else 0.03
         err = (got - want).abs().max(-1).values / want.abs().max()
         assert float(err[clear].max()) <= bar, (T, float(err[clear].max()))

@@ -145,8 +145,13 @@ def run(args):
             sec = timed(lambda: sops.gated_act(a, gu[:, :ff], gu[:, ff:], "relu"), it)
             record(kern, f"dopipel.gated_act.{tag}", sec, nbytes=T * ff * 6.0)
             hh = torch.randn(T, width, device=dev, dtype=dt)
-            sec = timed(lambda: sops.moe_route(hh, moe.router.data, moe.correction.data, moe.shared_gate.data, top), it)
-            record(kern, f"dopipel.moe_route.{tag}", sec, nbytes=T * width * 2.0 + (E + s["identity"] + 1) * width * 4.0)
+            def route():        # as the layer routes: many tokens take their logits from one fp32 product
+                logits = torch.mm(hh.float(), moe.router_rows().t()) if T >= moe.ROUTE_PRODUCT_MIN_TOKENS else None
+                return sops.moe_route(hh, moe.router.data, moe.correction.data, moe.shared_gate.data, top, logits)
+
+            sec = timed(route, it)
+            record(kern, f"dopipel.moe_route.{tag}", sec, nbytes=T * width * 2.0 + (E + s["identity"] + 1) * width * 4.0,
+                   note="prompt: cast + fp32 product + choice kernel; decode: one kernel")
             experts, weights, sg = sops.moe_route(hh, moe.router.data, moe.correction.data, moe.shared_gate.data, top)
             sec = timed(lambda: sops.moe_plan(experts, E), it)
             record(kern, f"dopipel.moe_plan.{tag}", sec, nbytes=T * top * 12.0, note="one workgroup")

@@ -118,7 +118,7 @@ def seq_lib():
         L.vla_seq_mingru_scratch_floats.restype = i64
         L.vla_seq_mingru_scan.argtypes = [p, i64, p, i64, p, i64, p, i64, p, p, p, p, i, i, i, i, p,
                                           i64, i, p]
-        L.vla_seq_moe_route.argtypes = [p, i64, p, p, p, p, p, p, i, i, i, i, i, p]
+        L.vla_seq_moe_route.argtypes = [p, i64, p, p, i64, p, p, p, p, p, i, i, i, i, i, p]
         L.vla_seq_moe_tile_rows.argtypes = []
         L.vla_seq_moe_plan.argtypes = [p, i, i, i, p, p, p, i, p]
         L.vla_seq_grouped_linear.argtypes = [p, i64, i, p, i64, p, p, p, i, i, i, i, i, p]

@@ -447,22 +447,27 @@ def mingru_scan(out: torch.Tensor, zp: torch.Tensor, up: torch.Tensor, gp: torch
 
 
 def moe_route(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor],
-              shared_gate_weight: Optional[torch.Tensor], top: int):
-    """-> experts int32 [T, top], weights fp32 [T, top], shared gate fp32 [T] or None."""
-    _gpu(h, router, correction, shared_gate_weight)
+              shared_gate_weight: Optional[torch.Tensor], top: int, logits: Optional[torch.Tensor] = None):
+    """-> experts int32 [T, top], weights fp32 [T, top], shared gate fp32 [T] or None.  logits
+    (fp32 [T, routed (+ 1, the shared gate's last)]): the router products, when the caller formed
+    them as one matrix product."""
+    _gpu(h, router, correction, shared_gate_weight, logits)
     T, W = h.shape
     N = router.shape[0]
     assert router.dtype == torch.float32 and router.is_contiguous() and router.shape[1] == W
     assert correction is None or (correction.dtype == torch.float32 and correction.numel() == N)
     assert shared_gate_weight is None or (shared_gate_weight.dtype == torch.float32 and shared_gate_weight.numel() == W)
+    if logits is not None:
+        assert logits.dtype == torch.float32 and logits.is_contiguous()
+        assert logits.shape == (T, N + (0 if shared_gate_weight is None else 1))
     experts = torch.empty((T, top), dtype=torch.int32, device=h.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=h.device)
     sg = None if shared_gate_weight is None else torch.empty((T, ), dtype=torch.float32, device=h.device)
     with torch.cuda.device(h.device):
         seq_check(_lib.seq_lib().vla_seq_moe_route(
-            h.data_ptr(), _rows(h, W), router.data_ptr(), _p(correction), _p(shared_gate_weight),
-            experts.data_ptr(), weights.data_ptr(), _p(sg), T, W, N, int(top), _dt(h.dtype), _stream(h.device)),
-            "moe_route")
+            h.data_ptr(), _rows(h, W), router.data_ptr(), _p(logits), 0 if logits is None else logits.shape[1],
+            _p(correction), _p(shared_gate_weight), experts.data_ptr(), weights.data_ptr(), _p(sg), T, W, N,
+            int(top), _dt(h.dtype), _stream(h.device)), "moe_route")
     return experts, weights, sg
 
 

@@ -376,7 +376,9 @@ __global__ __launch_bounds__(256, 2) void kv_attention_tile_kernel(
   const int b = blockIdx.z;
   const int row_blocks = 4 / head_waves;              // blocks of 32 query rows per workgroup
   const int tile_rows = kTile * row_blocks;
-  const int t_first = query_start_loc[b] + tile_rows * blockIdx.x;
+  // the last tiles of a run have the most keys to walk: they are dispatched first
+  const int tile_x = gridDim.x - 1 - blockIdx.x;
+  const int t_first = query_start_loc[b] + tile_rows * tile_x;
   const int n_tile = min(tile_rows, query_start_loc[b + 1] - t_first);
   if (n_tile <= 0) return;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
@@ -389,7 +391,7 @@ __global__ __launch_bounds__(256, 2) void kv_attention_tile_kernel(
   const int t0 = t_first + kTile * rb;
   const int nq = min(kTile, n_tile - kTile * rb);     // <= 0: no rows for this wave
   const bool active = h < g * group + group && nq > 0;
-  const int p_first = context_lens[b] + tile_rows * blockIdx.x, p_last = p_first + n_tile - 1;
+  const int p_first = context_lens[b] + tile_rows * tile_x, p_last = p_first + n_tile - 1;
   const int p0 = p_first + kTile * rb;                // this wave's first position
   const int pq = p0 + c;
   const int j_lo = window > 0 ? max(0, p_first - window + 1) : 0;

@@ -11,7 +11,7 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kKeep = 8;          // row elements a thread keeps in registers (rows up to 2048)
-constexpr int kMaxTaps = 16;
+constexpr int kMaxTaps = 32;
 
 template <class SY, class SO>
 __global__ __launch_bounds__(kThreads) void residual_norms_kernel(

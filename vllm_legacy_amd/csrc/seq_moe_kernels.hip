@@ -32,26 +32,33 @@ __device__ __forceinline__ float act_apply(float z, int act) {
   }
 }
 
+// One workgroup per token.  The logits come from the caller (a matrix product over many tokens) or
+// are formed here, a router row per wave at a time.
 template <class S>
 __global__ __launch_bounds__(256) void moe_route_kernel(
     const typename S::T* __restrict__ h, int64_t h_stride, const float* __restrict__ router,
-    const float* __restrict__ correction, const float* __restrict__ shared_gate_w,
-    int* __restrict__ experts, float* __restrict__ weights, float* __restrict__ shared_gate,
-    int width, int routed, int top) {
+    const float* __restrict__ logits, int64_t logits_stride, const float* __restrict__ correction,
+    const float* __restrict__ shared_gate_w, int* __restrict__ experts, float* __restrict__ weights,
+    float* __restrict__ shared_gate, int width, int routed, int top) {
   __shared__ float z[kMaxRouted + 1];
   const int t = blockIdx.x, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const typename S::T* hr = h + (int64_t)t * h_stride;
-  const int rows = routed + (shared_gate_w != nullptr ? 1 : 0);
-  for (int n = w; n < rows; n += 4) {
-    const float* wr = n < routed ? router + (int64_t)n * width : shared_gate_w;
-    float dot = 0.f;
-    for (int c = lane; c < width; c += kWave) dot += wr[c] * S::to_f32(hr[c]);
-    dot = wave_sum(dot);
-    if (lane == 0) z[n] = dot;
+  const bool gated = shared_gate != nullptr;
+  const int rows = routed + (gated ? 1 : 0);
+  if (logits != nullptr) {
+    for (int n = threadIdx.x; n < rows; n += 256) z[n] = logits[(int64_t)t * logits_stride + n];
+  } else {
+    const typename S::T* hr = h + (int64_t)t * h_stride;
+    for (int n = w; n < rows; n += 4) {
+      const float* wr = n < routed ? router + (int64_t)n * width : shared_gate_w;
+      float dot = 0.f;
+      for (int c = lane; c < width; c += kWave) dot += wr[c] * S::to_f32(hr[c]);
+      dot = wave_sum(dot);
+      if (lane == 0) z[n] = dot;
+    }
   }
   __syncthreads();
   if (w != 0) return;
-  if (shared_gate_w != nullptr && lane == 0) shared_gate[t] = 1.f / (1.f + expf(-z[routed]));
+  if (gated && lane == 0) shared_gate[t] = 1.f / (1.f + expf(-z[routed]));
   constexpr int PER = kMaxRouted / kWave;
   float s[PER], choice[PER];
   float mx = -INFINITY;
@@ -381,19 +388,22 @@ using namespace vla;
 using namespace vla::seq;
 
 extern "C" int vla_seq_moe_route(const void* h, int64_t h_stride, const float* router,
+                                 const float* logits, int64_t logits_stride,
                                  const float* correction, const float* shared_gate_weight,
                                  int* experts, float* weights, float* shared_gate, int num_tokens,
                                  int width, int routed, int top, int dtype, void* stream) {
   if (num_tokens == 0) return VLA_OK;
-  if (!h || !router || !experts || !weights || num_tokens < 0 || width <= 0 || routed <= 0 ||
-      routed > kMaxRouted || top <= 0 || top > routed || top > kWave || h_stride < width ||
-      (shared_gate_weight && !shared_gate))
+  const bool gated = shared_gate != nullptr;
+  if (!experts || !weights || num_tokens < 0 || width <= 0 || routed <= 0 || routed > kMaxRouted ||
+      top <= 0 || top > routed || top > kWave ||
+      (logits ? logits_stride < routed + (gated ? 1 : 0)
+              : (!h || !router || h_stride < width || (gated && !shared_gate_weight))))
     return VLA_ERR_ARG;
   return with_dtype(dtype, [&](auto s) {
     using S = decltype(s);
     moe_route_kernel<S><<<num_tokens, 256, 0, (hipStream_t)stream>>>(
-        (const typename S::T*)h, h_stride, router, correction, shared_gate_weight, experts, weights,
-        shared_gate, width, routed, top);
+        (const typename S::T*)h, h_stride, router, logits, logits_stride, correction,
+        shared_gate_weight, experts, weights, shared_gate, width, routed, top);
     VLA_SEQ_HIP_CHECK(hipGetLastError());
     return VLA_OK;
   });

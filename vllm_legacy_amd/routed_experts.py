@@ -6,7 +6,8 @@ largest s + correction are chosen and weighted by their s renormalized to sum 1.
 W_down act(W_up h).  An optional shared expert of the same form runs for every token, multiplied by
 sigmoid(w_sg . h).  The output is fp32 (the caller norms it and adds it to its stream).
 
-Execution (csrc/seq_moe_kernels.hip): route -> plan (pairs grouped by expert into row tiles) ->
+Execution (csrc/seq_moe_kernels.hip): route (the logits of a large step come from one fp32 matrix
+product) -> plan (pairs grouped by expert into row tiles) ->
 grouped up-projection with the activation fused (rows gathered from the tokens) -> grouped
 down-projection in fp32 -> combine (weighted sum per token in the order of its choices, identity
 experts and the shared expert added there).  Nothing synchronises with the host.
@@ -27,6 +28,9 @@ def mm_f32(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 
 class RoutedExperts(nn.Module):
+    # steps with at least this many tokens form the router logits as one matrix product; below,
+    # the routing kernel forms them itself (one launch)
+    ROUTE_PRODUCT_MIN_TOKENS = 256
 
     def __init__(self, width: int, num_experts: int, num_identity: int, top: int, expert_ff: int,
                  shared_ff: int = 0, act: str = "relu2", shared_act: Optional[str] = None,
@@ -38,6 +42,7 @@ class RoutedExperts(nn.Module):
         self.expert_ff, self.shared_ff, self.act = expert_ff, shared_ff, act
         self.shared_act = shared_act or act
         self.dtype = dtype
+        self._router_rows = None
         routed = num_experts + num_identity
 
         def par(shape, dt):
@@ -62,6 +67,7 @@ class RoutedExperts(nn.Module):
                 raise ValueError(f"{name}: shape {tuple(value.shape)}, expected {tuple(param.shape)}")
             param.data = value.to(param.dtype).to(dev).contiguous()
 
+        self._router_rows = None
         put(self.router, t["router"], "router")
         if "correction" in t:
             put(self.correction, t["correction"].reshape(routed), "correction")
@@ -73,11 +79,22 @@ class RoutedExperts(nn.Module):
             put(self.shared_down, t["shared.down"], "shared.down")
             put(self.shared_gate, t["shared.sg"].reshape(self.width), "shared.sg")
 
+    def router_rows(self) -> torch.Tensor:
+        """fp32 [routed (+ 1), width]: the router and, last, the shared expert's gate."""
+        if self._router_rows is None:
+            self._router_rows = torch.cat([self.router.data, self.shared_gate.data[None]], 0).contiguous() \
+                if self.shared_ff else self.router.data
+        return self._router_rows
+
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         """h [T, width] in the activation dtype -> fp32 [T, width]."""
         T = h.shape[0]
+        logits = None
+        if T >= self.ROUTE_PRODUCT_MIN_TOKENS:
+            # many tokens: the router rows (and the shared gate's) as one fp32 matrix product
+            logits = torch.mm(h if h.dtype == torch.float32 else h.float(), self.router_rows().t())
         experts, weights, sg = ops.moe_route(h, self.router.data, self.correction.data,
-                                             self.shared_gate.data if self.shared_ff else None, self.top)
+                                             self.shared_gate.data if self.shared_ff else None, self.top, logits)
         if self.num_experts:
             pair_row, row_token, tile_expert = ops.moe_plan(experts, self.num_experts)
             rows = row_token.numel()
