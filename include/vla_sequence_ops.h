@@ -260,6 +260,10 @@ int vla_seq_grouped_linear(void* out, int64_t out_stride, int out_dtype, const v
                            const int* tile_expert, int max_tiles, int n_out, int k_in, int act,
                            int dtype, void* stream);
 
+/* Form of the 16-bit product for tests: 0 = per shape, 1 = one-wave workgroups (decode steps),
+ * 2 = runs of tiles per workgroup (prompts). */
+int vla_seq_set_grouped_linear_form(int mode);
+
 /* out[t] (fp32 [T, width]) = sum_k weights[t, k] * (y[pair_row[t, k]] or, where pair_row is -1,
  * h[t]) + shared_gate[t] * shared_y[t] (shared_y null: none; shared_gate null: 1).  y, shared_y
  * fp32 rows of `width`. */

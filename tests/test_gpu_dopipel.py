@@ -421,6 +421,35 @@ def test_routed_experts(shape, dtype):
         assert float(err[clear].max()) <= bar, (T, float(err[clear].max()))
 
 
+@pytest.mark.parametrize("shape", [(64, 2, 0, 2, 64, 16), (128, 5, 1, 2, 64, 0), (64, 3, 0, 1, 48, 0)])
+@pytest.mark.parametrize("form", [1, 2])
+def test_grouped_products_in_every_form(shape, form):
+    """The 16-bit expert products in the form for decode steps and in the forms for prompts (runs of
+    tiles of one expert; through LDS where the inner size is a multiple of 64)."""
+    from vllm_legacy_amd import _seq_ops as ops
+    from vllm_legacy_amd.routed_experts import RoutedExperts
+    W, E, I, top, ff, sff = shape
+    mlp = R.moe_mlp(E, I, top, ff, sff)
+    cfg = R.make_config([R.mingru_layer(8, mlp)], width=W)
+    t = R.sub(R.make_weights(cfg, seed=5), "l0.mlp.")
+    layer = RoutedExperts(W, E, I, top, ff, sff, dtype=torch.bfloat16, device=DEV)
+    layer.set_weights(t)
+    tt = {k: v.to(F) for k, v in t.items()}
+    ops.set_grouped_linear_form(form)
+    try:
+        for T in (3, 70, 333):
+            h = rnd((T, W), T).to(torch.bfloat16)
+            want = R.moe_ff(h.to(F), tt, mlp)
+            s = torch.softmax(h.to(F) @ tt["router"].T, -1) + tt["correction"]
+            srt = torch.sort(s, -1, descending=True).values
+            clear = (srt[:, :top] - srt[:, 1:top + 1]).min(-1).values > 1e-3 if top < E + I else torch.ones(T, dtype=torch.bool)
+            got = layer(h.to(DEV)).cpu()
+            err = (got - want).abs().max(-1).values / want.abs().max()
+            assert float(err[clear].max()) <= 0.03, (T, float(err[clear].max()))
+    finally:
+        ops.set_grouped_linear_form(0)
+
+
 # ------------------------------------------------------------------------------------------------
 # whole models
 

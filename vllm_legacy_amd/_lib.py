@@ -59,7 +59,7 @@ SEQ_EXPORTS = [
     "vla_seq_rotary_kv_write", "vla_seq_kv_attention", "vla_seq_mingru_scratch_floats",
     "vla_seq_mingru_scan", "vla_seq_moe_route", "vla_seq_moe_tile_rows", "vla_seq_moe_plan",
     "vla_seq_grouped_linear", "vla_seq_moe_combine", "vla_seq_kv_attention_tiles_supported",
-    "vla_seq_kv_attention_tiles", "vla_seq_set_kv_attention_kernel",
+    "vla_seq_kv_attention_tiles", "vla_seq_set_kv_attention_kernel", "vla_seq_set_grouped_linear_form",
 ]
 _seq_lib = None
 
@@ -114,6 +114,7 @@ def seq_lib():
         L.vla_seq_kv_attention_tiles.argtypes = [p, i64, p, i64, p, i64, p, p, p, i, p, p, p, i, i, i,
                                                  i, i, i, i, i, i, i, f, i, p]
         L.vla_seq_set_kv_attention_kernel.argtypes = [i]
+        L.vla_seq_set_grouped_linear_form.argtypes = [i]
         L.vla_seq_mingru_scratch_floats.argtypes = [i, i, i]
         L.vla_seq_mingru_scratch_floats.restype = i64
         L.vla_seq_mingru_scan.argtypes = [p, i64, p, i64, p, i64, p, i64, p, p, p, p, i, i, i, i, p,

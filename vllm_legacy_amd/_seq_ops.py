@@ -507,6 +507,11 @@ def grouped_linear(out: torch.Tensor, a: torch.Tensor, row_token: Optional[torch
             tile_expert.data_ptr(), tiles, N, K, ACT[act], _dt(a.dtype), _stream(a.device)), "grouped_linear")
 
 
+def set_grouped_linear_form(mode: int) -> None:
+    """0: grouped_linear picks its 16-bit form per shape; 1: one-wave workgroups; 2: runs of tiles."""
+    seq_check(_lib.seq_lib().vla_seq_set_grouped_linear_form(mode), "set_grouped_linear_form")
+
+
 def moe_combine(out: torch.Tensor, y: torch.Tensor, pair_row: torch.Tensor, weights: torch.Tensor,
                 h: torch.Tensor, shared_y: Optional[torch.Tensor], shared_gate: Optional[torch.Tensor]) -> None:
     _gpu(out, y, pair_row, weights, h, shared_y, shared_gate)

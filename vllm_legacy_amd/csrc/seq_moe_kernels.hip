@@ -10,6 +10,8 @@
 //   moe_combine    per token: weighted sum of its experts' rows (a choice without a row is an
 //                  identity expert: the token's own input), plus the gated shared expert
 // A row's result does not depend on which other rows share its tile or on where the plan put it.
+#include <atomic>
+
 #include "seq_common.h"
 
 namespace vla {
@@ -17,6 +19,7 @@ namespace seq {
 namespace {
 
 constexpr int kTile = 32;
+std::atomic<int> g_grouped_form{0};
 constexpr int kMaxRouted = 512;   // experts a router chooses among, identity experts included
 
 __device__ __forceinline__ float act_apply(float z, int act) {
@@ -318,6 +321,114 @@ __global__ __launch_bounds__(256) void grouped_linear_mfma16_kernel(
   }
 }
 
+// The form for many tiles and k_in a multiple of 64: the activation rows of a run of tiles (up to
+// 128 rows) walk through LDS in chunks of 64 values, staged once for the four waves of the
+// workgroup (double-buffered, one barrier per chunk, loaded one chunk ahead); a wave's weight
+// fragments still come straight from memory (no other wave wants them), one 16-byte load per 16
+// values and 32 columns, used for every tile of the run.
+constexpr int kChunk = 64;
+constexpr int kARow = kChunk + 8;     // elements: 144-byte rows, 16 lanes' 16-byte reads fall into different banks
+
+template <class S, class SO, int C>
+__device__ __forceinline__ void grouped_run_lds(typename S::T* __restrict__ a_lds,
+                                                typename SO::T* __restrict__ out, int64_t out_stride,
+                                                const typename S::T* __restrict__ a, int64_t a_stride,
+                                                const int* __restrict__ row_token,
+                                                const typename S::T* __restrict__ wr, int first_tile, int n0,
+                                                int n_out, int k_in, int act, int hf, int c) {
+  using T = typename S::T;
+  const int tid = threadIdx.x;
+  // staging: C pieces of 16 bytes per thread and chunk; piece p = tid + 256 u is row p / 8, values 8 (p % 8) ..
+  const T* src[C];
+#pragma unroll
+  for (int u = 0; u < C; ++u) {
+    const int p = tid + 256 * u;
+    const int row = first_tile * kTile + p / 8;
+    const int tok = row_token != nullptr ? row_token[row] : row;
+    src[u] = tok < 0 ? nullptr : a + (int64_t)tok * a_stride + 8 * (p % 8);
+  }
+  u32x4 xa[C];
+  auto fetch = [&](int ch) {
+#pragma unroll
+    for (int u = 0; u < C; ++u)
+      xa[u] = src[u] != nullptr ? *reinterpret_cast<const u32x4*>(src[u] + ch * kChunk) : u32x4{0u, 0u, 0u, 0u};
+  };
+  auto land = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < C; ++u) {
+      const int p = tid + 256 * u;
+      *reinterpret_cast<u32x4*>(a_lds + (size_t)buf * 4 * kTile * kARow + (p / 8) * kARow + 8 * (p % 8)) = xa[u];
+    }
+  };
+  f32x16 acc[C];
+#pragma unroll
+  for (int r = 0; r < C; ++r)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[r][i] = 0.f;
+  const int chunks = k_in / kChunk;
+  fetch(0);
+  land(0);
+  if (chunks > 1) fetch(1);
+  __syncthreads();
+  for (int ch = 0; ch < chunks; ++ch) {
+    const T* tile = a_lds + (size_t)(ch & 1) * 4 * kTile * kARow + c * kARow + 8 * hf;
+    u32x4 wv[kChunk / 16];
+#pragma unroll
+    for (int ks = 0; ks < kChunk / 16; ++ks) wv[ks] = *reinterpret_cast<const u32x4*>(wr + ch * kChunk + 16 * ks);
+#pragma unroll
+    for (int ks = 0; ks < kChunk / 16; ++ks)
+#pragma unroll
+      for (int r = 0; r < C; ++r) {
+        const u32x4 av = *reinterpret_cast<const u32x4*>(tile + r * kTile * kARow + 16 * ks);
+        acc[r] = Mma16<S>::run(wv[ks], av, acc[r]);
+      }
+    if (ch + 1 < chunks) land((ch + 1) & 1);
+    if (ch + 2 < chunks) fetch(ch + 2);
+    __syncthreads();
+  }
+  if (n0 >= n_out) return;
+#pragma unroll
+  for (int r = 0; r < C; ++r) {
+    const int row = (first_tile + r) * kTile + c;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int n = n0 + (i & 3) + 8 * (i >> 2) + 4 * hf;
+      if (n < n_out) out[(int64_t)row * out_stride + n] = SO::from_f32(act_apply(acc[r][i], act));
+    }
+  }
+}
+
+template <class S, class SO>
+__global__ __launch_bounds__(256) void grouped_linear_lds_kernel(
+    typename SO::T* __restrict__ out, int64_t out_stride, const typename S::T* __restrict__ a,
+    int64_t a_stride, const int* __restrict__ row_token, const typename S::T* __restrict__ weight,
+    const int* __restrict__ tile_expert, int max_tiles, int n_out, int k_in, int act) {
+  __shared__ __align__(16) typename S::T a_lds[2 * 4 * kTile * kARow];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int hf = lane >> 5, c = lane & 31;
+  const int n0 = blockIdx.y * 128 + w * 32;        // waves past the last column still stage and wait
+  const int first = blockIdx.x * kRunTiles;
+  const int last = min(first + kRunTiles, max_tiles);
+  int i = first;
+  while (i < last) {
+    const int e = tile_expert[i];
+    if (e < 0) {
+      ++i;
+      continue;
+    }
+    int j = i + 1;
+    while (j < last && tile_expert[j] == e) ++j;
+    const typename S::T* wr = weight + ((int64_t)e * n_out + min(n0 + c, n_out - 1)) * k_in + 8 * hf;
+    switch (j - i) {
+      case 1: grouped_run_lds<S, SO, 1>(a_lds, out, out_stride, a, a_stride, row_token, wr, i, n0, n_out, k_in, act, hf, c); break;
+      case 2: grouped_run_lds<S, SO, 2>(a_lds, out, out_stride, a, a_stride, row_token, wr, i, n0, n_out, k_in, act, hf, c); break;
+      case 3: grouped_run_lds<S, SO, 3>(a_lds, out, out_stride, a, a_stride, row_token, wr, i, n0, n_out, k_in, act, hf, c); break;
+      default: grouped_run_lds<S, SO, 4>(a_lds, out, out_stride, a, a_stride, row_token, wr, i, n0, n_out, k_in, act, hf, c); break;
+    }
+    i = j;
+  }
+}
+
 // Any dtype and size, fp32 arithmetic: wave w of a workgroup takes eight rows of the tile, lane =
 // output column.
 template <class S, class SO>
@@ -442,7 +553,16 @@ extern "C" int vla_seq_grouped_linear(void* out, int64_t out_stride, int out_dty
         // few tiles (decode steps): the launch is bound by reading each expert's weights once, so
         // every (tile, 32 columns) is a one-wave workgroup of its own; many tiles: four waves
         // and runs of tiles that share the weight fragments
-        const bool few = (int64_t)max_tiles * ((n_out + 127) / 128) <= 1024;
+        const int form = g_grouped_form.load(std::memory_order_relaxed);
+        const bool few = form == 0 ? (int64_t)max_tiles * ((n_out + 127) / 128) <= 1024 : form == 1;
+        if (!few && k_in % kChunk == 0) {
+          grouped_linear_lds_kernel<S, SO>
+              <<<dim3((max_tiles + kRunTiles - 1) / kRunTiles, (n_out + 127) / 128), 256, 0, st>>>(
+                  (typename SO::T*)out, out_stride, (const T*)a, a_stride, row_token, (const T*)weight,
+                  tile_expert, max_tiles, n_out, k_in, act);
+          VLA_SEQ_HIP_CHECK(hipGetLastError());
+          return VLA_OK;
+        }
         const int waves = few ? 1 : 4, per = few ? 1 : kRunTiles;
         grouped_linear_mfma16_kernel<S, SO>
             <<<dim3((max_tiles + per - 1) / per, (n_out + 32 * waves - 1) / (32 * waves)), 64 * waves, 0, st>>>(
@@ -483,4 +603,12 @@ extern "C" int vla_seq_moe_combine(float* out, const float* y, const int* pair_r
     VLA_SEQ_HIP_CHECK(hipGetLastError());
     return VLA_OK;
   });
+}
+
+// 0: grouped_linear picks its 16-bit form per shape; 1: always one-wave workgroups; 2: always runs of
+// tiles (through LDS when k_in allows).  Tests run all.
+extern "C" int vla_seq_set_grouped_linear_form(int mode) {
+  if (mode < 0 || mode > 2) return VLA_ERR_ARG;
+  g_grouped_form.store(mode, std::memory_order_relaxed);
+  return VLA_OK;
 }
