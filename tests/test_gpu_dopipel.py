@@ -47,7 +47,7 @@ def configs():
         # more taps than some requests have tokens, no loop
         "taps": R.make_config([M(32, D(48)), A(2, 1, 32, mlp=E(4, 1, 2, 16, 16))], width=48, taps=6),
         # head sizes for the matrix-core kernels: multiples of 32, groups larger than a chunk
-        "mfma": R.make_config([A(10, 2, 32, vdim=64, mlp=D(64)), A(2, 1, 96, mlp=E(6, 1, 2, 32, 32)),
+        "mfma": R.make_config([A(10, 2, 32, vdim=64, mlp=D(64)), A(2, 1, 96, vdim=64, mlp=E(6, 1, 2, 32, 32)),
                                A(4, 4, 64, vdim=32, rot_dims=32, mlp=None)], width=128, loop=(0, 2, 2)),
     }
 
@@ -231,7 +231,7 @@ ATTN_SHAPES = [
     (6, 3, 8, 20, 8, "halves"),
     (2, 2, 40, 6, 0, "interleaved"),
     (10, 2, 32, 64, 32, "interleaved"),
-    (2, 1, 96, 96, 96, "interleaved"),
+    (2, 1, 96, 64, 64, "interleaved"),
     (8, 1, 64, 32, 32, "halves"),
     (5, 5, 128, 128, 64, "interleaved"),
     (2, 1, 32, 96, 32, "halves"),
@@ -257,7 +257,7 @@ def test_rotary_attention_prompt_portions_and_decoding(shape, dtype):
 def test_plain_and_matrix_core_kernels_agree():
     """bfloat16 through the kernel every dtype can take and through the matrix-core kernels."""
     from vllm_legacy_amd import _seq_ops as ops
-    H, G, D, V = 6, 2, 96, 64
+    H, G, D, V = 8, 2, 96, 64
     spec = attention_spec(H, G, D, V, 64, 1000.0)
     n = 101
     q, k, v, gate = (t.to(torch.bfloat16).float() for t in (rnd((n, H, D), 0), rnd((n, G, D), 1), rnd((n, G, V), 2), rnd((n, H), 3)))
@@ -380,7 +380,7 @@ MOE_SHAPES = [
     (64, 6, 1, 2, 24, 32),
     (40, 3, 0, 1, 20, 0),
     (64, 1, 2, 3, 16, 8),
-    (96, 12, 2, 2, 64, 96),
+    (96, 10, 3, 2, 48, 80),
     (72, 5, 3, 4, 130, 0),
     (50, 4, 1, 2, 9, 7),       # sizes the matrix-core product does not take: the plain one runs
     (72, 2, 0, 1, 40, 0),      # multiples of 8 but not of 16: the narrower matrix-core product
